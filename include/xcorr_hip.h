@@ -1,0 +1,232 @@
+/*
+ * xcorr_hip.h - C ABI of libxcorr_hip.so: definition-based 2D cross-correlation
+ * on AMD MI355X (gfx950), hand-written HIP kernels.
+ *
+ * The entry points replace the launcher functions of the reference's
+ * repo/cross-corr/src/kernels.cuh (the `run_*` templates, lines 41-283) one for
+ * one: plain pointers to caller-owned device memory, sizes, tuning integers and a
+ * stream. Like the reference launchers they neither allocate nor copy nor
+ * synchronise; the launch is asynchronous on `stream` (NULL = the default stream).
+ *
+ * Conventions shared by every compute entry point
+ *   - matrices are dense row-major `rows x cols`; the matrices of an array are
+ *     contiguous (reference matrix.hpp:590-595); left and right matrices have the
+ *     same size (validate.hpp:94-101 assumes it);
+ *   - every result matrix is `(2*rows-1) x (2*cols-1)`; element (oy, ox) is the
+ *     shift (oy-(rows-1), ox-(cols-1)):
+ *         out[oy][ox] = sum over (y, x) of left[y+sy][x+sx] * right[y][x]
+ *     which equals the reference host result validate.hpp:117-132 with
+ *     ref = left, target = right;
+ *   - return value: XCORR_OK or an error code; the message is available from
+ *     xcorr_last_error(). Where the reference launcher throws
+ *     std::runtime_error for a tuning value (e.g.
+ *     naive_shuffle_multirow_both.cu:645-665) the entry point returns
+ *     XCORR_ERR_INVALID_ARGUMENT with an equivalent message. Nothing throws
+ *     across this boundary;
+ *   - a tuning field of xcorr_params set to 0 selects the library's tuned default;
+ *   - after a successful launch the geometry actually used is available from
+ *     xcorr_last_launch() (reference kernel_args.hpp:9-33, a process-global that
+ *     is not thread-safe there either).
+ */
+#ifndef XCORR_HIP_H
+#define XCORR_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XCORR_OK 0
+#define XCORR_ERR_INVALID_ARGUMENT 1 /* bad tuning value or shape (reference: std::runtime_error) */
+#define XCORR_ERR_RUNTIME 2          /* a HIP runtime call failed (reference: CUCH, cuda_helpers.cuh:13-24) */
+#define XCORR_ERR_UNSUPPORTED 3      /* combination this build has no kernel for */
+
+/* reference row_distribution.cuh:9-13 */
+#define XCORR_DIST_DEFAULT 0
+#define XCORR_DIST_NONE 1
+#define XCORR_DIST_RECTANGLE 2
+#define XCORR_DIST_TRIANGLE 3
+
+/* variants of the warp-per-overlap family (reference naive_warp_per_shift.cu) */
+#define XCORR_WPO_BASE 0              /* run_ccn_warp_per_shift, kernels.cuh:99-107 */
+#define XCORR_WPO_SIMPLE_INDEXING 1   /* run_ccn_warp_per_shift_simple_indexing, kernels.cuh:109-117 */
+#define XCORR_WPO_WORK_DISTRIBUTION 2 /* run_ccn_warp_per_shift_work_distribution, kernels.cuh:119-128 */
+
+/*
+ * Tuning integers, named after the reference's per-algorithm JSON keys
+ * (one_to_one.hpp:739-741, n_to_m.hpp:321-325, n_to_m.hpp:475-479, ...). The
+ * reference counts 32-lane warps; this library runs 64-lane wavefronts and maps
+ * a request onto the nearest gfx950 specialisation, see xcorr_last_launch().
+ * Upper limits are the reference's release limits (CMakeLists.txt:16-46); larger
+ * values are rejected as there.
+ */
+typedef struct xcorr_params {
+    unsigned warps_per_thread_block;         /* <= 32 */
+    unsigned shifts_per_thread_block;        /* <= 32, warp-per-overlap family */
+    unsigned rows_per_thread;                /* split-row: max overlap rows per worker (JSON rows_per_thread / rows_per_warp) */
+    unsigned distribution_type;              /* XCORR_DIST_* */
+    unsigned shifts_per_thread;              /* grouped-overlap, <= 8 */
+    unsigned left_rows_per_iteration;        /* grouped-overlap <= 8, combined kernels <= 4 */
+    unsigned right_matrices_per_thread;      /* <= 8, combined kernels <= 4 */
+    unsigned left_matrices_per_thread;       /* <= 8, combined kernels <= 4 */
+    unsigned shifts_per_thread_right_matrix; /* combined kernels, <= 4 */
+    unsigned warp_per_overlap_variant;       /* XCORR_WPO_* */
+    /* gfx950 tile geometry, no counterpart in the reference; 0 = tuned default */
+    unsigned x_shifts_per_thread;            /* adjacent x shifts one lane accumulates: 4 or 8 */
+    unsigned lanes_x;                        /* lanes of a wavefront laid along x shifts (power of two) */
+    unsigned lanes_y;                        /* lanes laid along y shifts; the rest are laid over matrices */
+    unsigned reserved[3];
+} xcorr_params;
+
+/* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the
+ * template parameters each launcher records, e.g. naive_shuffle_multirow_both.cu:488-522). */
+typedef struct xcorr_launch_record {
+    char kernel[64];
+    unsigned block[3];
+    unsigned grid[3];
+    unsigned shared_mem_bytes;
+    unsigned y_shifts_per_thread;
+    unsigned x_shifts_per_thread;
+    unsigned left_matrices_per_thread;
+    unsigned right_matrices_per_thread;
+    unsigned lanes_x, lanes_y, lanes_left, lanes_right; /* how the 64 lanes are laid out */
+    unsigned waves_x, waves_y;
+    unsigned rows_per_worker;  /* left rows one work item reduces over */
+    unsigned distribution_type;
+    unsigned uses_atomics;     /* 1: partial sums are added with float atomics into a zeroed output */
+} xcorr_launch_record;
+
+typedef struct xcorr_device_info {
+    char name[128];
+    char arch[32];
+    int compute_units;
+    int clock_khz;        /* engine clock */
+    int memory_clock_khz;
+    int memory_bus_bits;
+    int lds_bytes_per_block;
+    size_t global_mem_bytes;
+    double fp32_vector_peak_tflops; /* CUs x 4 SIMD x 16 lanes x 2 (packed) x 2 FLOP x clock */
+    double fp64_vector_peak_tflops; /* CUs x 4 SIMD x 16 lanes x 2 FLOP x clock */
+} xcorr_device_info;
+
+/* ---- status ---- */
+const char *xcorr_last_error(void);
+int xcorr_last_launch(xcorr_launch_record *out);
+int xcorr_device_info_get(xcorr_device_info *out);
+const char *xcorr_version(void);
+
+/* ---- memory / queue shims: the C++ host never includes the HIP headers.
+ * They stand in for the reference's cuda_helpers.cuh:26-97 (cuda_malloc,
+ * cuda_memcpy_to_device, cuda_memcpy_from_device, cuda_memset, cuda_free),
+ * allocator.cuh:16-86 (pinned host memory) and stopwatch.hpp:236-301 (events). ---- */
+int xcorr_malloc(void **dev_ptr, size_t bytes);
+int xcorr_free(void *dev_ptr);
+int xcorr_memset_async(void *dev_ptr, int value, size_t bytes, void *stream);
+int xcorr_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes);
+int xcorr_memcpy_d2h(void *host_dst, const void *dev_src, size_t bytes);
+int xcorr_memcpy_h2d_async(void *dev_dst, const void *host_src, size_t bytes, void *stream);
+int xcorr_memcpy_d2h_async(void *host_dst, const void *dev_src, size_t bytes, void *stream);
+int xcorr_host_alloc_pinned(void **host_ptr, size_t bytes);
+int xcorr_host_free(void *host_ptr);
+int xcorr_stream_create(void **stream);
+int xcorr_stream_destroy(void *stream);
+int xcorr_stream_sync(void *stream);
+int xcorr_device_sync(void);
+int xcorr_event_create(void **event);
+int xcorr_event_record(void *event, void *stream);
+int xcorr_event_sync(void *event);
+int xcorr_event_elapsed_ms(void *start, void *stop, float *ms);
+int xcorr_event_destroy(void *event);
+
+/* ---- compute entry points ---- */
+
+/* Overlap-wise: one thread per shift, serial loop over the overlap.
+ * Replaces run_cross_corr_naive_original (kernels.cuh:41-51, naive_original.cu:130-161):
+ * `n_left` = subregions_per_pic, `batch` = batch_size. Right matrix b*n_left + i is
+ * correlated with left matrix i; the result has the right matrix's index. */
+int xcorr_overlap_wise_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                           unsigned n_left, unsigned batch, void *stream);
+int xcorr_overlap_wise_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                           unsigned n_left, unsigned batch, void *stream);
+
+/* Warp-per-overlap: one wavefront per shift, lanes stride the overlap, DPP reduction.
+ * Replaces run_ccn_warp_per_shift, run_ccn_warp_per_shift_simple_indexing and
+ * run_ccn_warp_per_shift_work_distribution (kernels.cuh:99-128). One pair.
+ * Uses p->shifts_per_thread_block, p->warp_per_overlap_variant and, for the
+ * work-distribution variant (caller zeroes `out` first, as one_to_one.hpp:476-489),
+ * p->rows_per_thread and p->distribution_type. */
+int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                               const xcorr_params *p, void *stream);
+int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                               const xcorr_params *p, void *stream);
+
+/* Sliding-window base: every lane owns adjacent x shifts of one output row.
+ * Replaces run_ccn_shuffle (kernels.cuh:65-73). One pair. Uses p->warps_per_thread_block. */
+int xcorr_shuffle_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                      const xcorr_params *p, void *stream);
+int xcorr_shuffle_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                      const xcorr_params *p, void *stream);
+
+/* Split-row: the overlap rows of an output row are split over several workers of at
+ * most p->rows_per_thread rows each, partial sums are added atomically.
+ * Replaces run_ccn_shuffle_work_distribution<DIST> (kernels.cuh:75-85). One pair.
+ * THE CALLER ZEROES `out` FIRST (reference one_to_one.hpp:276-277). */
+int xcorr_split_row_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                        const xcorr_params *p, void *stream);
+int xcorr_split_row_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                        const xcorr_params *p, void *stream);
+
+/* Grouped-overlap: every lane accumulates p->shifts_per_thread adjacent y shifts.
+ * Replaces run_ccn_shuffle_multirow_both (kernels.cuh:185-195). One pair.
+ * `out` need not be zeroed: when the launcher splits the reduction to fill the
+ * device it clears `out` itself on `stream` first. */
+int xcorr_grouped_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                              const xcorr_params *p, void *stream);
+int xcorr_grouped_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                              const xcorr_params *p, void *stream);
+
+/* Multi-matrix-right: one left matrix against n_right right matrices, each lane
+ * reuses a left value for p->right_matrices_per_thread right matrices.
+ * Replaces run_ccn_shuffle_multimat_right (kernels.cuh:87-97) when
+ * p->rows_per_thread == 0 and run_ccn_shuffle_multimat_right_work_distribution<DIST>
+ * (kernels.cuh:130-142; caller zeroes `out`) otherwise. Result i = left x right i. */
+int xcorr_multimat_right_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                             unsigned n_right, const xcorr_params *p, void *stream);
+int xcorr_multimat_right_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                             unsigned n_right, const xcorr_params *p, void *stream);
+
+/* Multi-matrix-right x grouped-overlap.
+ * Replaces run_ccn_shuffle_one_to_many_multirow_both_multimat_right (kernels.cuh:221-234).
+ * Extension: n_left > 1 runs the n_to_mn mode in one launch, left l against the
+ * right matrices [l*n_right, (l+1)*n_right) (the de-interleaved order of
+ * n_to_mn.hpp:165-172), result index = right index. `out` need not be zeroed. */
+int xcorr_multimat_right_grouped_f32(const float *left, const float *right, float *out, unsigned cols,
+                                     unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                     void *stream);
+int xcorr_multimat_right_grouped_f64(const double *left, const double *right, double *out, unsigned cols,
+                                     unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                     void *stream);
+
+/* Multi-matrix-both: all n_left x n_right pairs, result index l*n_right + r, split-row.
+ * Replaces run_ccn_shuffle_n_to_m_multimat_both_work_distribution<DIST>
+ * (kernels.cuh:163-176). THE CALLER ZEROES `out` FIRST (n_to_m.hpp:341). */
+int xcorr_multimat_both_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                            unsigned n_left, unsigned n_right, const xcorr_params *p, void *stream);
+int xcorr_multimat_both_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                            unsigned n_left, unsigned n_right, const xcorr_params *p, void *stream);
+
+/* Multi-matrix-both x grouped-overlap.
+ * Replaces run_ccn_n_to_m_shuffle_multirow_both_multimat_both (kernels.cuh:236-250).
+ * `out` need not be zeroed. */
+int xcorr_multimat_both_grouped_f32(const float *left, const float *right, float *out, unsigned cols,
+                                    unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                    void *stream);
+int xcorr_multimat_both_grouped_f64(const double *left, const double *right, double *out, unsigned cols,
+                                    unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                    void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,198 @@
+// Host-side planner and launcher of the sliding-window engine: picks a compiled
+// specialisation for a request, decides how the reduction over left rows is split
+// into work items, clears the output when it splits on its own, launches and
+// records the geometry.
+#include <cmath>
+
+#include "engine_registry.hpp"
+
+namespace xcorr {
+
+static int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
+            cus = prop.multiProcessorCount;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)); }
+
+// Relative cost of running the request on a specialisation: work issued for partial
+// overlaps at tile edges, lanes idling over matrices that do not exist, and LDS read
+// time when a tile has too little register reuse. Hints scale the cost so the nearest
+// specialisation wins without excluding the others.
+static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
+    double waste_x = (double)(rq.W + s.TXW()) / rq.W;
+    double waste_y = (double)(rq.H + s.TYW()) / rq.H;
+    int nu = rq.group_m > 0 ? rq.group_m : rq.nU;
+    double util_v = (double)rq.nV / ((double)ceil_div(rq.nV, s.NVB()) * s.NVB());
+    double util_u = (double)nu / ((double)ceil_div(nu, s.NUB()) * s.NUB());
+    int vk = 16 / s.elem_bytes;
+    double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
+    double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
+    double lds = 8.0 * reads / fmas * 1.15; // LDS cycles per VALU cycle with four SIMDs sharing one LDS
+    double cost = waste_x * waste_y / (util_v * util_u) * (lds > 1.0 ? lds : 1.0);
+    // very small grids cannot fill the device: prefer narrower tiles then
+    if (rq.y_shifts > 1) cost *= 1.0 + 0.25 * log2_ratio(s.A, rq.y_shifts);
+    if (rq.left_mats) cost *= 1.0 + 0.25 * log2_ratio(s.NV, rq.left_mats);
+    if (rq.right_mats) cost *= 1.0 + 0.25 * log2_ratio(s.NU, rq.right_mats);
+    if (rq.waves) cost *= 1.0 + 0.05 * log2_ratio(s.WX * s.WY, rq.waves);
+    return cost;
+}
+
+int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
+    int count = 0;
+    const EngineSpec *specs = rq.elem_bytes == 4 ? engine_specs_f32(&count) : engine_specs_f64(&count);
+    const EngineSpec *best = nullptr;
+    double best_cost = 0;
+    for (int i = 0; i < count; ++i) {
+        const EngineSpec &s = specs[i];
+        if ((rq.y_shifts == 1) != (s.A == 1)) continue; // one-output-row families vs grouped families
+        if (rq.group_m > 0 && s.NVB() != 1) continue;
+        if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
+        if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
+        if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
+        double c = spec_cost(s, rq);
+        if (!best || c < best_cost) {
+            best = &s;
+            best_cost = c;
+        }
+    }
+    if (!best)
+        return fail(XCORR_ERR_UNSUPPORTED, "%s: no compiled specialisation matches x_shifts_per_thread=%u lanes_x=%u lanes_y=%u",
+                    rq.family, rq.x_shifts, rq.lanes_x, rq.lanes_y);
+    plan.spec = best;
+    const int Sx = 2 * rq.W - 1, Sy = 2 * rq.H - 1;
+    plan.ntx = ceil_div(Sx, best->TXB());
+    plan.nty = ceil_div(Sy, best->TYB());
+    plan.nvg = ceil_div(rq.nV, best->NVB());
+    plan.nug = ceil_div(rq.group_m > 0 ? rq.group_m : rq.nU, best->NUB());
+    const long tiles = (long)plan.ntx * plan.nty * plan.nvg * plan.nug;
+
+    int dist = rq.dist == XCORR_DIST_NONE ? 0 : rq.dist == XCORR_DIST_RECTANGLE ? 1 : rq.dist == XCORR_DIST_TRIANGLE ? 2 : -1;
+    int rc = (int)rq.rows_per_worker;
+    if (rq.caller_zeroes) {
+        // split-row contract (reference one_to_one.hpp:276-288): zeroed output, atomics
+        if (dist < 0) dist = 1; // the reference's default is "rectangle" (one_to_one.hpp:232)
+        if (rc <= 0) rc = best->RL;
+        if (dist == 0) rc = rq.H;
+        plan.atomic = 1;
+        plan.zero_fill = false;
+    } else {
+        if (rc <= 0 && rq.may_split) {
+            const long target = 16L * device_cus();
+            long chunks_wanted = (target + tiles - 1) / tiles;
+            if (chunks_wanted > 1) {
+                rc = ceil_div(rq.H, (int)chunks_wanted);
+                rc = ceil_div(rc, best->RL) * best->RL;
+            }
+        }
+        if (rc <= 0 || rc >= rq.H || !rq.may_split) {
+            rc = rq.H;
+            dist = 0;
+            plan.atomic = 0;
+            plan.zero_fill = false;
+        } else {
+            if (dist <= 0) dist = 2;
+            plan.atomic = 1;
+            plan.zero_fill = true;
+        }
+    }
+    if (rc > rq.H) rc = rq.H;
+    plan.rows_per_chunk = rc;
+    plan.dist = dist;
+
+    // workers along y: (y tile, chunk) pairs
+    int max_chunks = 0;
+    long total_chunks = 0;
+    for (int ty = 0; ty < plan.nty; ++ty) {
+        int syb = -(rq.H - 1) + ty * best->TYB();
+        int lo = syb > 0 ? syb : 0;
+        int hi = syb + best->TYB() - 1 + rq.H;
+        if (hi > rq.H) hi = rq.H;
+        int n = ceil_div(hi - lo, rc);
+        if (n > max_chunks) max_chunks = n;
+        total_chunks += n;
+    }
+    if (dist == 0)
+        plan.nworkers_y = plan.nty;
+    else if (dist == 1)
+        plan.nworkers_y = plan.nty * max_chunks;
+    else
+        plan.nworkers_y = (int)total_chunks;
+    long grid = (long)plan.nvg * plan.nug * plan.nworkers_y * plan.ntx;
+    if (grid <= 0 || grid > 0x7fffffffL) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: grid of %ld blocks is out of range", rq.family, grid);
+    plan.grid = (unsigned)grid;
+    return XCORR_OK;
+}
+
+template <typename T>
+static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStream_t stream) {
+    EngineArgs<T> a;
+    a.V = static_cast<const T *>(rq.V);
+    a.U = static_cast<const T *>(rq.U);
+    a.out = static_cast<T *>(rq.out);
+    a.W = rq.W;
+    a.H = rq.H;
+    a.nV = rq.nV;
+    a.nU = rq.nU;
+    a.group_m = rq.group_m;
+    a.rows_per_chunk = plan.rows_per_chunk;
+    a.dist = plan.dist;
+    a.atomic = plan.atomic;
+    a.ntx = plan.ntx;
+    a.nty = plan.nty;
+    a.nworkers_y = plan.nworkers_y;
+    a.nvg = plan.nvg;
+    a.nug = plan.nug;
+    if (plan.zero_fill) {
+        size_t n = (size_t)(2 * rq.W - 1) * (2 * rq.H - 1) * (rq.group_m > 0 ? (size_t)rq.nU : (size_t)rq.nV * rq.nU);
+        size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
+        if (blocks > 65536) blocks = 65536;
+        zero_fill_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a.out, n);
+        XCORR_HIP(hipGetLastError());
+    }
+    XCORR_HIP(plan.spec->launch(&a, plan.grid, stream));
+    return XCORR_OK;
+}
+
+int run_engine(const EngineRequest &rq, hipStream_t stream) {
+    EnginePlan plan;
+    int rc = plan_engine(rq, plan);
+    if (rc != XCORR_OK) return rc;
+    rc = rq.elem_bytes == 4 ? launch_typed<float>(rq, plan, stream) : launch_typed<double>(rq, plan, stream);
+    if (rc != XCORR_OK) return rc;
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "%s/%s", rq.family, plan.spec->name);
+    rec.block[0] = plan.spec->threads;
+    rec.block[1] = rec.block[2] = 1;
+    rec.grid[0] = plan.grid;
+    rec.grid[1] = rec.grid[2] = 1;
+    rec.shared_mem_bytes = plan.spec->lds_bytes;
+    rec.y_shifts_per_thread = plan.spec->A;
+    rec.x_shifts_per_thread = plan.spec->B;
+    rec.left_matrices_per_thread = plan.spec->NV;
+    rec.right_matrices_per_thread = plan.spec->NU;
+    rec.lanes_x = plan.spec->LX;
+    rec.lanes_y = plan.spec->LY;
+    rec.lanes_left = plan.spec->LV;
+    rec.lanes_right = plan.spec->LU;
+    rec.waves_x = plan.spec->WX;
+    rec.waves_y = plan.spec->WY;
+    rec.rows_per_worker = plan.rows_per_chunk;
+    rec.distribution_type = plan.dist == 0 ? XCORR_DIST_NONE : plan.dist == 1 ? XCORR_DIST_RECTANGLE : XCORR_DIST_TRIANGLE;
+    rec.uses_atomics = plan.atomic;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+} // namespace xcorr

@@ -1,0 +1,91 @@
+// Table of compiled engine specialisations and the host-side planner that maps a
+// request (sizes, matrix counts, the reference's tuning integers) onto one of them.
+//
+// The reference instantiates every value of every tuning integer up to a compile-time
+// limit (CMakeLists.txt:16-46, about six hours of build). Here a short list of
+// gfx950-tuned tiles is compiled and a request is mapped onto the nearest one; the
+// geometry actually used is reported through xcorr_last_launch().
+#pragma once
+
+#include "engine.hpp"
+#include "xcorr_common.hpp"
+
+namespace xcorr {
+
+struct EngineSpec {
+    const char *name;
+    int elem_bytes; // 4 or 8
+    int A, B, K, NV, NU;
+    int LX, LY, LV, LU;
+    int WX, WY, RL, KBX;
+    int lds_bytes;
+    int threads;
+    // launches the kernel; `args` points at an EngineArgs<T> of the matching type
+    hipError_t (*launch)(const void *args, unsigned grid, hipStream_t stream);
+    int TXW() const { return LX * B; }
+    int TYW() const { return LY * A; }
+    int TXB() const { return TXW() * WX; }
+    int TYB() const { return TYW() * WY; }
+    int NVB() const { return LV * NV; }
+    int NUB() const { return LU * NU; }
+};
+
+template <class C>
+hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
+    using T = typename C::value_type;
+    static bool attr_set = false;
+    if (!attr_set && C::LDS_BYTES > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&engine_kernel<C>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    engine_kernel<C><<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
+    return hipGetLastError();
+}
+
+template <class C>
+constexpr EngineSpec make_spec(const char *name) {
+    return EngineSpec{name,   (int)sizeof(typename C::value_type),
+                      C::A,   C::B,
+                      C::K,   C::NV,
+                      C::NU,  C::LX,
+                      C::LY,  C::LV,
+                      C::LU,  C::WX,
+                      C::WY,  C::RL,
+                      C::KBX, C::LDS_BYTES,
+                      C::NT,  &launch_engine<C>};
+}
+
+// defined in engine_f32.hip / engine_f64.hip
+const EngineSpec *engine_specs_f32(int *count);
+const EngineSpec *engine_specs_f64(int *count);
+
+// What a family asks of the engine.
+struct EngineRequest {
+    const char *family;
+    int elem_bytes;
+    const void *V, *U;
+    void *out;
+    int W, H, nV, nU;
+    int group_m;          // see EngineArgs
+    // hints (0 = none). y_shifts == 1 selects the one-output-row-per-lane specialisations.
+    unsigned y_shifts, x_shifts, left_mats, right_mats, lanes_x, lanes_y, waves;
+    unsigned rows_per_worker; // 0 = planner decides
+    unsigned dist;            // XCORR_DIST_*
+    bool caller_zeroes;       // true: split-row contract, output arrives zeroed, always accumulate atomically
+    bool may_split;           // planner may split the reduction and clear the output itself
+};
+
+struct EnginePlan {
+    const EngineSpec *spec;
+    int ntx, nty, nworkers_y, nvg, nug;
+    int rows_per_chunk, dist, atomic;
+    bool zero_fill;
+    unsigned grid;
+};
+
+int plan_engine(const EngineRequest &rq, EnginePlan &plan);
+int run_engine(const EngineRequest &rq, hipStream_t stream);
+
+} // namespace xcorr

@@ -1,0 +1,269 @@
+// Overlap-wise and warp-per-overlap kernel families for gfx950 wavefronts.
+//
+// overlap-wise      : one thread per shift, serial loop over the overlap straight from
+//                     global memory (the definition; the reference's starting point,
+//                     naive_original.cu:36-102).
+// warp-per-overlap  : one 64-lane wavefront per shift; lanes stride the overlap and the
+//                     partial sums are combined with DPP row operations (no LDS, no
+//                     ds_bpermute), replacing the 32-lane cg::reduce of
+//                     naive_warp_per_shift.cu:21-244.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "xcorr_common.hpp"
+
+namespace xcorr {
+
+// ------------------------------------------------------------------ DPP wave reduction
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double v) {
+    unsigned long long bits = __builtin_bit_cast(unsigned long long, v);
+    int lo = (int)(unsigned)bits, hi = (int)(unsigned)(bits >> 32);
+    lo = __builtin_amdgcn_update_dpp(0, lo, CTRL, ROW_MASK, 0xf, false);
+    hi = __builtin_amdgcn_update_dpp(0, hi, CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(double, ((unsigned long long)(unsigned)hi << 32) | (unsigned)lo);
+}
+
+// Sum over the 64 lanes of a wavefront; the total is valid in lane 63.
+template <typename T>
+__device__ __forceinline__ T wave_sum_to_lane63(T v) {
+    v += dpp_move<0xB1, 0xf>(v);  // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E, 0xf>(v);  // quad_perm [2,3,0,1]
+    v += dpp_move<0x141, 0xf>(v); // row_half_mirror
+    v += dpp_move<0x140, 0xf>(v); // row_mirror: every lane of a 16-lane row holds the row sum
+    v += dpp_move<0x142, 0xa>(v); // row_bcast:15 into rows 1 and 3
+    v += dpp_move<0x143, 0xc>(v); // row_bcast:31 into rows 2 and 3
+    return v;
+}
+
+__device__ __forceinline__ void atomic_add_simple(float *p, float v) { unsafeAtomicAdd(p, v); }
+__device__ __forceinline__ void atomic_add_simple(double *p, double v) { unsafeAtomicAdd(p, v); }
+
+// ------------------------------------------------------------------ overlap-wise
+// Thread (x, y) of the strip of n_left result matrices laid side by side computes one
+// shift, for every one of the `batch` right matrices paired with its left matrix.
+template <typename T>
+__global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__ left, const T *__restrict__ right,
+                                                            T *__restrict__ out, int W, int H, int n_left, int batch) {
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
+    const int strip_x = blockIdx.x * blockDim.x + threadIdx.x;
+    const int oy = blockIdx.y * blockDim.y + threadIdx.y;
+    const int region = strip_x / Sx;
+    if (region >= n_left || oy >= Sy) return;
+    const int ox = strip_x - region * Sx;
+    const int sx = ox - (W - 1), sy = oy - (H - 1);
+    const int xl_lo = sx > 0 ? sx : 0, xl_hi = W + sx < W ? W + sx : W;
+    const int yl_lo = sy > 0 ? sy : 0, yl_hi = H + sy < H ? H + sy : H;
+    const size_t in_area = (size_t)W * H, out_area = (size_t)Sx * Sy;
+    const T *l = left + region * in_area;
+    for (int b = 0; b < batch; ++b) {
+        const size_t mat = (size_t)b * n_left + region;
+        const T *r = right + mat * in_area;
+        T sum = T(0);
+        for (int yl = yl_lo; yl < yl_hi; ++yl) {
+            const T *lrow = l + (size_t)yl * W;
+            const T *rrow = r + (size_t)(yl - sy) * W - sx;
+            for (int xl = xl_lo; xl < xl_hi; ++xl) sum += rrow[xl] * lrow[xl];
+        }
+        out[mat * out_area + (size_t)oy * Sx + ox] = sum;
+    }
+}
+
+template <typename T>
+int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
+                     unsigned batch, hipStream_t stream) {
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_left == 0 || batch == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
+    dim3 block(64, 4);
+    unsigned long long strip = (unsigned long long)Sx * n_left;
+    if (strip > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "strip of %u result matrices is too wide", n_left);
+    dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y);
+    overlap_wise_kernel<T><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch);
+    XCORR_HIP(hipGetLastError());
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "overlap_wise/%s", sizeof(T) == 4 ? "f32" : "f64");
+    rec.block[0] = block.x, rec.block[1] = block.y, rec.block[2] = 1;
+    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = 1;
+    rec.y_shifts_per_thread = rec.x_shifts_per_thread = 1;
+    rec.left_matrices_per_thread = 1;
+    rec.right_matrices_per_thread = batch;
+    rec.distribution_type = XCORR_DIST_NONE;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+// ------------------------------------------------------------------ warp-per-overlap
+// Dense ("triangle") packing of split-row workers: output row r has
+// ceil(overlap_rows(r) / max_rows) workers, numbered consecutively over rows.
+__host__ __device__ inline unsigned wpo_overlap_rows(unsigned row, unsigned H) { return row < H ? row + 1 : 2 * H - 1 - row; }
+__host__ __device__ inline unsigned wpo_workers(unsigned row, unsigned H, unsigned max_rows) {
+    return (wpo_overlap_rows(row, H) + max_rows - 1) / max_rows;
+}
+// number of workers of output rows [0, n) for n <= H (ascending half)
+__host__ __device__ inline unsigned long long wpo_prefix_ascending(unsigned n, unsigned R) {
+    unsigned long long q = n / R, rem = n % R;
+    return (unsigned long long)R * q * (q + 1) / 2 + rem * (q + 1);
+}
+// number of workers of output rows [0, n), 0 <= n <= 2H-1
+__host__ __device__ inline unsigned long long wpo_prefix(unsigned n, unsigned H, unsigned R) {
+    if (n <= H) return wpo_prefix_ascending(n, R);
+    // rows H .. n-1 mirror rows H-2 .. 2H-1-n
+    unsigned m = n - H; // count of descending rows taken
+    return wpo_prefix_ascending(H, R) + (wpo_prefix_ascending(H - 1, R) - wpo_prefix_ascending(H - 1 - m, R));
+}
+
+struct WpoWork {
+    unsigned row, idx, per_row;
+};
+
+template <int DIST>
+__device__ __forceinline__ WpoWork wpo_distribute(unsigned worker, unsigned max_rows, unsigned H) {
+    const unsigned Sy = 2 * H - 1;
+    WpoWork w;
+    if (DIST == 0) {
+        w.row = worker;
+        w.idx = 0;
+        w.per_row = worker < Sy ? 1u : 0u;
+    } else if (DIST == 1) {
+        w.row = worker % Sy;
+        w.idx = worker / Sy;
+        w.per_row = wpo_workers(w.row, H, max_rows);
+    } else {
+        // largest row whose prefix is <= worker
+        unsigned lo = 0, hi = Sy; // prefix(lo) <= worker < prefix(hi) unless worker is surplus
+        if (worker >= wpo_prefix(Sy, H, max_rows)) {
+            w.row = Sy;
+            w.idx = 0;
+            w.per_row = 0;
+            return w;
+        }
+        while (hi - lo > 1) {
+            unsigned mid = (lo + hi) / 2;
+            if (wpo_prefix(mid, H, max_rows) <= worker)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        w.row = lo;
+        w.idx = worker - (unsigned)wpo_prefix(lo, H, max_rows);
+        w.per_row = wpo_workers(lo, H, max_rows);
+    }
+    return w;
+}
+
+// VARIANT 0: lanes stride the flattened overlap; 1: row loop, lanes stride the columns;
+// 2: as 0 but the rows of a shift are split over workers (DIST) and added atomically.
+template <typename T, int VARIANT, int DIST>
+__global__ __launch_bounds__(1024) void warp_per_overlap_kernel(const T *__restrict__ left, const T *__restrict__ right,
+                                                                 T *__restrict__ out, int W, int H, unsigned max_rows) {
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
+    const int lane = threadIdx.x;
+    const int ox = blockIdx.x * blockDim.y + threadIdx.y;
+    int oy = blockIdx.y;
+    unsigned part = 0, parts = 1;
+    if (VARIANT == 2) {
+        WpoWork w = wpo_distribute<DIST>(blockIdx.y, max_rows, (unsigned)H);
+        if (w.idx >= w.per_row) return;
+        oy = (int)w.row;
+        part = w.idx;
+        parts = w.per_row;
+    }
+    if (ox >= Sx || oy >= Sy) return;
+    const int sx = ox - (W - 1), sy = oy - (H - 1);
+    // overlap in right-matrix coordinates
+    const int xr_lo = sx < 0 ? -sx : 0, xr_hi = W - sx < W ? W - sx : W;
+    int yr_lo = sy < 0 ? -sy : 0, yr_hi = H - sy < H ? H - sy : H;
+    if (VARIANT == 2) {
+        const int rows_all = yr_hi - yr_lo;
+        const int per = (rows_all + (int)parts - 1) / (int)parts;
+        yr_lo += (int)part * per;
+        if (yr_lo + per < yr_hi) yr_hi = yr_lo + per;
+    }
+    const int ow = xr_hi - xr_lo, oh = yr_hi - yr_lo;
+    T sum = T(0);
+    if (VARIANT == 1) {
+        for (int yr = yr_lo; yr < yr_hi; ++yr) {
+            const T *rrow = right + (size_t)yr * W;
+            const T *lrow = left + (size_t)(yr + sy) * W + sx;
+            for (int xr = xr_lo + lane; xr < xr_hi; xr += 64) sum += lrow[xr] * rrow[xr];
+        }
+    } else if (oh > 0 && ow > 0) {
+        const unsigned total = (unsigned)ow * (unsigned)oh;
+        for (unsigned i = lane; i < total; i += 64) {
+            const unsigned row = i / (unsigned)ow, col = i - row * (unsigned)ow;
+            const int yr = yr_lo + (int)row, xr = xr_lo + (int)col;
+            sum += left[(size_t)(yr + sy) * W + (xr + sx)] * right[(size_t)yr * W + xr];
+        }
+    }
+    sum = wave_sum_to_lane63(sum);
+    if (lane == 63) {
+        T *p = out + (size_t)oy * Sx + ox;
+        if (VARIANT == 2)
+            atomic_add_simple(p, sum);
+        else
+            *p = sum;
+    }
+}
+
+template <typename T>
+int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params &p,
+                         hipStream_t stream) {
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    // reference limit: naive_warp_per_shift.cu:316-318 (32 warps of 32 lanes per block)
+    if ((rc = check_limit("shifts per thread block", p.shifts_per_thread_block, 32))) return rc;
+    if (p.warp_per_overlap_variant > XCORR_WPO_WORK_DISTRIBUTION)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "Unknown warp-per-overlap variant %u", p.warp_per_overlap_variant);
+    if (p.distribution_type > XCORR_DIST_TRIANGLE) return fail(XCORR_ERR_INVALID_ARGUMENT, "Unknown distribution %u", p.distribution_type);
+    unsigned spb = p.shifts_per_thread_block ? p.shifts_per_thread_block : 8; // reference default one_to_one.hpp:415
+    if (spb > 16) spb = 16; // a block holds at most 16 wavefronts of 64 lanes
+    const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
+    dim3 block(64, spb);
+    unsigned grid_y = Sy;
+    unsigned max_rows = p.rows_per_thread ? p.rows_per_thread : 3; // reference default rows_per_warp, one_to_one.hpp:458
+    unsigned dist = p.distribution_type == XCORR_DIST_DEFAULT ? XCORR_DIST_RECTANGLE : p.distribution_type;
+    const int variant = (int)p.warp_per_overlap_variant;
+    if (variant == 2) {
+        if (dist == XCORR_DIST_NONE)
+            grid_y = Sy;
+        else if (dist == XCORR_DIST_RECTANGLE)
+            grid_y = Sy * ((rows + max_rows - 1) / max_rows);
+        else
+            grid_y = (unsigned)wpo_prefix(Sy, rows, max_rows);
+    }
+    dim3 grid((Sx + spb - 1) / spb, grid_y);
+    const int W = (int)cols, H = (int)rows;
+    if (variant == 0)
+        warp_per_overlap_kernel<T, 0, 0><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
+    else if (variant == 1)
+        warp_per_overlap_kernel<T, 1, 0><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
+    else if (dist == XCORR_DIST_NONE)
+        warp_per_overlap_kernel<T, 2, 0><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
+    else if (dist == XCORR_DIST_RECTANGLE)
+        warp_per_overlap_kernel<T, 2, 1><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
+    else
+        warp_per_overlap_kernel<T, 2, 2><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
+    XCORR_HIP(hipGetLastError());
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "warp_per_overlap/%s_v%d", sizeof(T) == 4 ? "f32" : "f64", variant);
+    rec.block[0] = block.x, rec.block[1] = block.y, rec.block[2] = 1;
+    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = 1;
+    rec.y_shifts_per_thread = rec.x_shifts_per_thread = 1;
+    rec.left_matrices_per_thread = rec.right_matrices_per_thread = 1;
+    rec.rows_per_worker = variant == 2 ? max_rows : rows;
+    rec.distribution_type = variant == 2 ? dist : XCORR_DIST_NONE;
+    rec.uses_atomics = variant == 2;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+} // namespace xcorr

@@ -1,0 +1,366 @@
+// extern "C" surface of libxcorr_hip.so: status, memory / queue shims and the
+// compute entry points that stand in for the reference launchers (kernels.cuh:41-283).
+#include "engine_registry.hpp"
+#include "simple_kernels.hpp"
+#include "xcorr_common.hpp"
+
+using namespace xcorr;
+
+static hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+extern "C" {
+
+// ------------------------------------------------------------------ status
+const char *xcorr_last_error(void) { return error_buffer(); }
+
+const char *xcorr_version(void) { return "xcorr_hip 0.1 (gfx950)"; }
+
+int xcorr_last_launch(xcorr_launch_record *out) {
+    if (!out) return fail(XCORR_ERR_INVALID_ARGUMENT, "null record pointer");
+    if (!have_last_launch()) return fail(XCORR_ERR_INVALID_ARGUMENT, "No kernel launch");
+    *out = last_launch();
+    return XCORR_OK;
+}
+
+int xcorr_device_info_get(xcorr_device_info *out) {
+    if (!out) return fail(XCORR_ERR_INVALID_ARGUMENT, "null info pointer");
+    int dev = 0;
+    XCORR_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    XCORR_HIP(hipGetDeviceProperties(&prop, dev));
+    memset(out, 0, sizeof(*out));
+    snprintf(out->name, sizeof(out->name), "%s", prop.name);
+    snprintf(out->arch, sizeof(out->arch), "%s", prop.gcnArchName);
+    out->compute_units = prop.multiProcessorCount;
+    out->clock_khz = prop.clockRate;
+    out->memory_clock_khz = prop.memoryClockRate;
+    out->memory_bus_bits = prop.memoryBusWidth;
+    out->lds_bytes_per_block = (int)prop.sharedMemPerBlock;
+    out->global_mem_bytes = prop.totalGlobalMem;
+    double lanes_per_s = (double)prop.multiProcessorCount * 4.0 * 16.0 * (double)prop.clockRate * 1e3;
+    out->fp32_vector_peak_tflops = lanes_per_s * 2.0 * 2.0 / 1e12;
+    out->fp64_vector_peak_tflops = lanes_per_s * 2.0 / 1e12;
+    return XCORR_OK;
+}
+
+// ------------------------------------------------------------------ shims
+int xcorr_malloc(void **dev_ptr, size_t bytes) {
+    if (!dev_ptr) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    XCORR_HIP(hipMalloc(dev_ptr, bytes));
+    return XCORR_OK;
+}
+int xcorr_free(void *dev_ptr) {
+    XCORR_HIP(hipFree(dev_ptr));
+    return XCORR_OK;
+}
+int xcorr_memset_async(void *dev_ptr, int value, size_t bytes, void *stream) {
+    XCORR_HIP(hipMemsetAsync(dev_ptr, value, bytes, as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes) {
+    XCORR_HIP(hipMemcpy(dev_dst, host_src, bytes, hipMemcpyHostToDevice));
+    return XCORR_OK;
+}
+int xcorr_memcpy_d2h(void *host_dst, const void *dev_src, size_t bytes) {
+    XCORR_HIP(hipMemcpy(host_dst, dev_src, bytes, hipMemcpyDeviceToHost));
+    return XCORR_OK;
+}
+int xcorr_memcpy_h2d_async(void *dev_dst, const void *host_src, size_t bytes, void *stream) {
+    XCORR_HIP(hipMemcpyAsync(dev_dst, host_src, bytes, hipMemcpyHostToDevice, as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_memcpy_d2h_async(void *host_dst, const void *dev_src, size_t bytes, void *stream) {
+    XCORR_HIP(hipMemcpyAsync(host_dst, dev_src, bytes, hipMemcpyDeviceToHost, as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_host_alloc_pinned(void **host_ptr, size_t bytes) {
+    if (!host_ptr) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    XCORR_HIP(hipHostMalloc(host_ptr, bytes, hipHostMallocDefault));
+    return XCORR_OK;
+}
+int xcorr_host_free(void *host_ptr) {
+    XCORR_HIP(hipHostFree(host_ptr));
+    return XCORR_OK;
+}
+int xcorr_stream_create(void **stream) {
+    if (!stream) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    hipStream_t s;
+    XCORR_HIP(hipStreamCreate(&s)); // default priority only
+    *stream = s;
+    return XCORR_OK;
+}
+int xcorr_stream_destroy(void *stream) {
+    XCORR_HIP(hipStreamDestroy(as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_stream_sync(void *stream) {
+    XCORR_HIP(hipStreamSynchronize(as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_device_sync(void) {
+    XCORR_HIP(hipDeviceSynchronize());
+    XCORR_HIP(hipGetLastError());
+    return XCORR_OK;
+}
+int xcorr_event_create(void **event) {
+    if (!event) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    hipEvent_t e;
+    XCORR_HIP(hipEventCreate(&e));
+    *event = e;
+    return XCORR_OK;
+}
+int xcorr_event_record(void *event, void *stream) {
+    XCORR_HIP(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_event_sync(void *event) {
+    XCORR_HIP(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+    return XCORR_OK;
+}
+int xcorr_event_elapsed_ms(void *start, void *stop, float *ms) {
+    if (!ms) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    XCORR_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return XCORR_OK;
+}
+int xcorr_event_destroy(void *event) {
+    XCORR_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return XCORR_OK;
+}
+
+} // extern "C"
+
+// ------------------------------------------------------------------ compute
+namespace {
+
+const xcorr_params zero_params = {};
+
+const xcorr_params &params_or_default(const xcorr_params *p) { return p ? *p : zero_params; }
+
+int check_dist(unsigned d) {
+    if (d > XCORR_DIST_TRIANGLE) return fail(XCORR_ERR_INVALID_ARGUMENT, "Unknown distribution %u", d);
+    return XCORR_OK;
+}
+
+// warps of the reference are 32 lanes wide; a wavefront holds two of them
+unsigned waves_from_warps(unsigned warps) { return warps == 0 ? 0 : (warps + 1) / 2; }
+
+EngineRequest base_request(const char *family, int elem_bytes, const void *left, const void *right, void *out,
+                           unsigned cols, unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params &p) {
+    EngineRequest rq = {};
+    rq.family = family;
+    rq.elem_bytes = elem_bytes;
+    rq.V = left;
+    rq.U = right;
+    rq.out = out;
+    rq.W = (int)cols;
+    rq.H = (int)rows;
+    rq.nV = (int)n_left;
+    rq.nU = (int)n_right;
+    rq.x_shifts = p.x_shifts_per_thread;
+    rq.lanes_x = p.lanes_x;
+    rq.lanes_y = p.lanes_y;
+    rq.waves = waves_from_warps(p.warps_per_thread_block);
+    rq.dist = p.distribution_type;
+    return rq;
+}
+
+template <typename T>
+int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
+                 void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    EngineRequest rq = base_request("shuffle", sizeof(T), left, right, out, cols, rows, 1, 1, p);
+    rq.y_shifts = 1;
+    rq.left_mats = rq.right_mats = 1;
+    rq.dist = XCORR_DIST_NONE;
+    rq.may_split = false;
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int split_row_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
+                   void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("split_row", sizeof(T), left, right, out, cols, rows, 1, 1, p);
+    rq.y_shifts = 1;
+    rq.left_mats = rq.right_mats = 1;
+    rq.rows_per_worker = p.rows_per_thread;
+    rq.caller_zeroes = true;
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
+                 void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_limit("shifts per thread", p.shifts_per_thread, Limits::shifts_per_thread))) return rc;
+    if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::left_rows))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);
+    rq.y_shifts = p.shifts_per_thread == 1 ? 2 : p.shifts_per_thread; // 0 = planner's choice among the grouped tiles
+    if (rq.y_shifts == 0) rq.y_shifts = 0;
+    rq.rows_per_worker = p.rows_per_thread;
+    rq.may_split = true;
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_right,
+                        const xcorr_params *pp, void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no right matrices");
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("multimat_right", sizeof(T), left, right, out, cols, rows, 1, n_right, p);
+    rq.y_shifts = 1;
+    rq.left_mats = 1;
+    rq.right_mats = p.right_matrices_per_thread;
+    if (p.rows_per_thread > 0) { // the work-distribution launcher
+        rq.rows_per_worker = p.rows_per_thread;
+        rq.caller_zeroes = true;
+    } else {
+        rq.dist = XCORR_DIST_NONE;
+        rq.may_split = false;
+    }
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int multimat_right_grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
+                                unsigned n_right, const xcorr_params *pp, void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_limit("shifts per thread per right matrix", p.shifts_per_thread_right_matrix, Limits::combined))) return rc;
+    if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::combined))) return rc;
+    if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::combined))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("multimat_right_grouped", sizeof(T), left, right, out, cols, rows, n_left,
+                                    n_left * n_right, p);
+    rq.group_m = n_left > 1 ? (int)n_right : 0;
+    if (n_left == 1) rq.nU = (int)n_right;
+    rq.y_shifts = p.shifts_per_thread_right_matrix == 1 ? 2 : p.shifts_per_thread_right_matrix;
+    rq.left_mats = 1;
+    rq.right_mats = p.right_matrices_per_thread;
+    rq.rows_per_worker = p.rows_per_thread;
+    rq.may_split = true;
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int multimat_both_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
+                       unsigned n_right, const xcorr_params *pp, void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_limit("left matrices per thread", p.left_matrices_per_thread, Limits::left_matrices))) return rc;
+    if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("multimat_both", sizeof(T), left, right, out, cols, rows, n_left, n_right, p);
+    rq.y_shifts = 1;
+    rq.left_mats = p.left_matrices_per_thread;
+    rq.right_mats = p.right_matrices_per_thread;
+    rq.rows_per_worker = p.rows_per_thread;
+    if (rq.dist == XCORR_DIST_DEFAULT) rq.dist = XCORR_DIST_TRIANGLE; // reference default, n_to_m.hpp:325
+    rq.caller_zeroes = true;
+    return run_engine(rq, as_stream(stream));
+}
+
+template <typename T>
+int multimat_both_grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
+                               unsigned n_right, const xcorr_params *pp, void *stream) {
+    const xcorr_params &p = params_or_default(pp);
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if ((rc = check_limit("shifts per thread per right matrix", p.shifts_per_thread_right_matrix, Limits::combined))) return rc;
+    if ((rc = check_limit("left matrices per thread", p.left_matrices_per_thread, Limits::combined))) return rc;
+    if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::combined))) return rc;
+    if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::combined))) return rc;
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    EngineRequest rq = base_request("multimat_both_grouped", sizeof(T), left, right, out, cols, rows, n_left, n_right, p);
+    rq.y_shifts = p.shifts_per_thread_right_matrix == 1 ? 2 : p.shifts_per_thread_right_matrix;
+    rq.left_mats = p.left_matrices_per_thread;
+    rq.right_mats = p.right_matrices_per_thread;
+    rq.rows_per_worker = p.rows_per_thread;
+    rq.may_split = true;
+    return run_engine(rq, as_stream(stream));
+}
+
+} // namespace
+
+extern "C" {
+
+int xcorr_overlap_wise_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                           unsigned n_left, unsigned batch, void *stream) {
+    return run_overlap_wise<float>(left, right, out, cols, rows, n_left, batch, as_stream(stream));
+}
+int xcorr_overlap_wise_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                           unsigned n_left, unsigned batch, void *stream) {
+    return run_overlap_wise<double>(left, right, out, cols, rows, n_left, batch, as_stream(stream));
+}
+
+int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                               const xcorr_params *p, void *stream) {
+    return run_warp_per_overlap<float>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+}
+int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                               const xcorr_params *p, void *stream) {
+    return run_warp_per_overlap<double>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+}
+
+#define XCORR_PAIR_ENTRY(NAME, IMPL)                                                                              \
+    int NAME##_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,               \
+                   const xcorr_params *p, void *stream) {                                                         \
+        return IMPL<float>(left, right, out, cols, rows, p, stream);                                              \
+    }                                                                                                             \
+    int NAME##_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,            \
+                   const xcorr_params *p, void *stream) {                                                         \
+        return IMPL<double>(left, right, out, cols, rows, p, stream);                                             \
+    }
+
+XCORR_PAIR_ENTRY(xcorr_shuffle, shuffle_impl)
+XCORR_PAIR_ENTRY(xcorr_split_row, split_row_impl)
+XCORR_PAIR_ENTRY(xcorr_grouped_overlap, grouped_impl)
+
+int xcorr_multimat_right_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                             unsigned n_right, const xcorr_params *p, void *stream) {
+    return multimat_right_impl<float>(left, right, out, cols, rows, n_right, p, stream);
+}
+int xcorr_multimat_right_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                             unsigned n_right, const xcorr_params *p, void *stream) {
+    return multimat_right_impl<double>(left, right, out, cols, rows, n_right, p, stream);
+}
+
+#define XCORR_NM_ENTRY(NAME, IMPL)                                                                                \
+    int NAME##_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,               \
+                   unsigned n_left, unsigned n_right, const xcorr_params *p, void *stream) {                      \
+        return IMPL<float>(left, right, out, cols, rows, n_left, n_right, p, stream);                             \
+    }                                                                                                             \
+    int NAME##_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,            \
+                   unsigned n_left, unsigned n_right, const xcorr_params *p, void *stream) {                      \
+        return IMPL<double>(left, right, out, cols, rows, n_left, n_right, p, stream);                            \
+    }
+
+XCORR_NM_ENTRY(xcorr_multimat_right_grouped, multimat_right_grouped_impl)
+XCORR_NM_ENTRY(xcorr_multimat_both, multimat_both_impl)
+XCORR_NM_ENTRY(xcorr_multimat_both_grouped, multimat_both_grouped_impl)
+
+} // extern "C"

@@ -1,0 +1,75 @@
+// Shared host-side pieces of libxcorr_hip.so: error state, last-launch record,
+// parameter validation against the reference's limits.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "../../include/xcorr_hip.h"
+
+namespace xcorr {
+
+// ---- error state (one message per thread) ----
+inline char *error_buffer() {
+    static thread_local char buf[512] = "";
+    return buf;
+}
+
+inline int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+inline int hip_check(hipError_t e, const char *what) {
+    if (e == hipSuccess) return XCORR_OK;
+    // same information as the reference's CUCH macro (cuda_helpers.cuh:13-24)
+    return fail(XCORR_ERR_RUNTIME, "HIP error %d (%s: %s) in %s", (int)e, hipGetErrorName(e), hipGetErrorString(e), what);
+}
+
+#define XCORR_HIP(call)                                  \
+    do {                                                 \
+        int _rc = ::xcorr::hip_check((call), #call);     \
+        if (_rc != XCORR_OK) return _rc;                 \
+    } while (0)
+
+// ---- last launch record (process-global, like reference kernel_args.cpp:7-19) ----
+inline xcorr_launch_record &last_launch() {
+    static xcorr_launch_record rec;
+    return rec;
+}
+inline bool &have_last_launch() {
+    static bool have = false;
+    return have;
+}
+
+// Release limits of the reference build (CMakeLists.txt:16-46).
+struct Limits {
+    static constexpr unsigned warps_per_block = 32;             // every launcher, e.g. naive_shuffle_multirow_both.cu:645
+    static constexpr unsigned shifts_per_thread = 8;            // SHUFFLE_MULTIROW_BOTH_SHIFTS_PER_THREAD_LIMIT
+    static constexpr unsigned left_rows = 8;                    // SHUFFLE_MULTIROW_BOTH_LEFT_ROWS_LIMIT
+    static constexpr unsigned right_matrices = 8;               // SHUFFLE_MULTIMAT_RIGHT_RIGHT_MATRICES_PER_THREAD_LIMIT
+    static constexpr unsigned left_matrices = 8;                // SHUFFLE_N_TO_M_MULTIMAT_BOTH_LEFT_MATRICES_PER_THREAD_LIMIT
+    static constexpr unsigned combined = 4;                     // the 4/4/4(/4) limits of the combined kernels
+};
+
+inline int check_limit(const char *what, unsigned value, unsigned limit) {
+    if (value > limit) return fail(XCORR_ERR_INVALID_ARGUMENT, "Too many %s: %u (max %u)", what, value, limit);
+    return XCORR_OK;
+}
+
+inline int check_shape(const void *left, const void *right, const void *out, unsigned cols, unsigned rows) {
+    if (!left || !right || !out) return fail(XCORR_ERR_INVALID_ARGUMENT, "null device pointer");
+    if (cols == 0 || rows == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "empty matrix: %u x %u", rows, cols);
+    // result indices are 32-bit in the kernels' per-matrix arithmetic
+    if (cols > 16384 || rows > 16384) return fail(XCORR_ERR_INVALID_ARGUMENT, "matrix too large: %u x %u (max 16384)", rows, cols);
+    return XCORR_OK;
+}
+
+} // namespace xcorr

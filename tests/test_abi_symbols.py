@@ -1,0 +1,65 @@
+"""CPU-only: the C ABI library loads without a GPU and exports every symbol that
+include/xcorr_hip.h declares; argument validation that needs no device works."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from conftest import load_package
+
+
+def declared_symbols():
+    xc = load_package()
+    text = open(xc.HEADER_PATH).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(xcorr_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_surface():
+    names = declared_symbols()
+    for family in ["overlap_wise", "warp_per_overlap", "shuffle", "split_row", "grouped_overlap", "multimat_right",
+                   "multimat_right_grouped", "multimat_both", "multimat_both_grouped"]:
+        assert f"xcorr_{family}_f32" in names and f"xcorr_{family}_f64" in names
+    assert len(names) >= 40
+
+
+def test_library_exports_every_declared_symbol():
+    xc = load_package()
+    if not os.path.exists(xc.LIB_PATH):
+        pytest.fail(f"{xc.LIB_PATH} not built")
+    lib = xc.lib()
+    for name in declared_symbols():
+        assert hasattr(lib, name), name
+
+
+def test_python_struct_mirrors_match_header_field_order():
+    xc = load_package()
+    text = open(xc.HEADER_PATH).read()
+    body = re.search(r"typedef struct xcorr_params \{(.*?)\} xcorr_params;", text, flags=re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    fields = re.findall(r"unsigned\s+([a-z_]+)(?:\[\d+\])?;", body)
+    assert fields == [f[0] for f in xc.Params._fields_]
+
+
+def test_argument_errors_without_a_device():
+    xc = load_package()
+    lib = xc.lib()
+    p = xc.make_params(shifts_per_thread=9)
+    dummy = ctypes.c_void_p(16)
+    rc = lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None)
+    assert rc == 1
+    assert b"Too many shifts per thread: 9 (max 8)" in lib.xcorr_last_error()
+    p = xc.make_params(warps_per_thread_block=33)
+    assert lib.xcorr_shuffle_f32(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None) == 1
+    assert b"Too many warps per thread block: 33 (max 32)" in lib.xcorr_last_error()
+    assert lib.xcorr_grouped_overlap_f32(None, dummy, dummy, 8, 8, None, None) == 1
+    assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 0, 8, None, None) == 1
+    p = xc.make_params(distribution_type=7)
+    assert lib.xcorr_split_row_f64(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None) == 1
+    assert b"Unknown distribution" in lib.xcorr_last_error()
+    p = xc.make_params(right_matrices_per_thread=5)
+    assert lib.xcorr_multimat_both_grouped_f32(dummy, dummy, dummy, 8, 8, 2, 2, ctypes.byref(p), None) == 1
+    rec = xc.LaunchRecord()
+    assert lib.xcorr_last_launch(ctypes.byref(rec)) == 1
+    assert b"No kernel launch" in lib.xcorr_last_error()

@@ -1,0 +1,241 @@
+"""GPU parity: every kernel family, called through the C ABI, against the CPU oracle on
+the same seeded inputs.
+
+Bars: integer-valued inputs (every product and sum exact) must match bit for bit in
+fp32 and fp64; real-valued inputs must match the oracle to a relative Frobenius error
+of 1e-5 (fp32) / 1e-12 (fp64), the tolerances of the build's brief. The GPU kernels add
+the same products in a different order than the oracle's sequential loop, so real-valued
+results are not expected to be bit-identical (nor are the reference's own kernels).
+"""
+import numpy as np
+import pytest
+
+from conftest import load_package
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+SHAPES = [(1, 1), (1, 7), (6, 1), (3, 5), (16, 16), (17, 33), (33, 17), (64, 64), (70, 130)]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def ints(rng, shape, dtype, amp=4):
+    return rng.integers(-amp, amp + 1, size=shape).astype(dtype)
+
+
+def rel_frob(a, b):
+    a = a.astype(np.float64).ravel()
+    b = b.astype(np.float64).ravel()
+    den = np.linalg.norm(b)
+    return np.linalg.norm(a - b) / (den if den > 0 else 1.0)
+
+
+def check(got, exp, exact, what):
+    assert got.shape == exp.shape, what
+    assert np.isfinite(got).all(), f"{what}: unwritten or non-finite output elements"
+    if exact:
+        bad = np.argwhere(got != exp)
+        assert bad.size == 0, f"{what}: {len(bad)} elements differ, first {bad[:3].tolist()}"
+    else:
+        err = rel_frob(got, exp)
+        assert err <= TOL[got.dtype], f"{what}: rel frobenius {err:.3e}"
+
+
+ONE_TO_ONE_CASES = [
+    ("overlap_wise", {}),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="base")),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="base", shifts_per_thread_block=3)),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="simple_indexing", shifts_per_thread_block=32)),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="none")),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="rectangle", rows_per_thread=3)),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="triangle", rows_per_thread=5)),
+    ("shuffle", {}),
+    ("shuffle", dict(warps_per_thread_block=4)),
+    ("split_row", dict(distribution_type="none")),
+    ("split_row", dict(distribution_type="rectangle", rows_per_thread=10)),
+    ("split_row", dict(distribution_type="triangle", rows_per_thread=4)),
+    ("split_row", dict(distribution_type="triangle", rows_per_thread=1)),
+    ("grouped_overlap", {}),
+    ("grouped_overlap", dict(shifts_per_thread=4, left_rows_per_iteration=3, warps_per_thread_block=8)),
+    ("grouped_overlap", dict(shifts_per_thread=8)),
+    ("grouped_overlap", dict(shifts_per_thread=1)),
+    ("grouped_overlap", dict(shifts_per_thread=8, rows_per_thread=16)),
+    ("grouped_overlap", dict(shifts_per_thread=4, rows_per_thread=7, distribution_type="rectangle")),
+    ("multimat_right", {}),
+    ("multimat_right_grouped", {}),
+    ("multimat_both", {}),
+    ("multimat_both_grouped", {}),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("family,kw", ONE_TO_ONE_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_one_to_one_all_families(oracle, dtype, family, kw):
+    xc = load_package()
+    rng = np.random.default_rng(100)
+    for shape in SHAPES:
+        say("one_to_one", family, kw, np.dtype(dtype).name, shape)
+        left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
+        exp = oracle.one_to_one(left, right)
+        got = xc.run(family, left, right, 1, params=xc.make_params(**kw))
+        check(got, exp, True, f"{family} {kw} {shape} int")
+        left = rng.standard_normal(shape).astype(dtype)
+        right = rng.random(shape).astype(dtype)
+        exp = oracle.one_to_one(left, right)
+        got = xc.run(family, left, right, 1, params=xc.make_params(**kw))
+        check(got, exp, False, f"{family} {kw} {shape} real")
+
+
+ONE_TO_MANY_CASES = [
+    ("multimat_right", {}),
+    ("multimat_right", dict(right_matrices_per_thread=1)),
+    ("multimat_right", dict(right_matrices_per_thread=8, warps_per_thread_block=4)),
+    ("multimat_right", dict(right_matrices_per_thread=2, rows_per_thread=10, distribution_type="rectangle")),
+    ("multimat_right", dict(right_matrices_per_thread=4, rows_per_thread=3, distribution_type="triangle")),
+    ("multimat_right_grouped", {}),
+    ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=4, right_matrices_per_thread=4, left_rows_per_iteration=4)),
+    ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=2, right_matrices_per_thread=2, rows_per_thread=16)),
+    ("multimat_both", dict(left_matrices_per_thread=1, right_matrices_per_thread=4)),
+    ("multimat_both_grouped", {}),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("family,kw", ONE_TO_MANY_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_one_to_many(oracle, dtype, family, kw):
+    xc = load_package()
+    rng = np.random.default_rng(200)
+    for shape, n_right in [((5, 9), 1), ((16, 16), 3), ((33, 20), 7), ((64, 64), 19)]:
+        say("one_to_many", family, kw, np.dtype(dtype).name, shape, n_right)
+        left = ints(rng, (1,) + shape, dtype)
+        right = ints(rng, (n_right,) + shape, dtype)
+        exp = oracle.one_to_many(left, right)
+        got = xc.run(family, left, right, n_right, n_left=1, n_right=n_right, params=xc.make_params(**kw))
+        check(got, exp, True, f"{family} {kw} {shape}x{n_right} int")
+        left = rng.standard_normal((1,) + shape).astype(dtype)
+        right = rng.standard_normal((n_right,) + shape).astype(dtype)
+        exp = oracle.one_to_many(left, right, threads=4)
+        got = xc.run(family, left, right, n_right, n_left=1, n_right=n_right, params=xc.make_params(**kw))
+        check(got, exp, False, f"{family} {kw} {shape}x{n_right} real")
+
+
+def test_overlap_wise_batches(oracle):
+    """run_cross_corr_naive_original's (subregions_per_pic, batch_size) layout: right matrix
+    b*n + i pairs with left i, i.e. the n_to_mn file order of validate.hpp:264-269."""
+    xc = load_package()
+    rng = np.random.default_rng(300)
+    for dtype in (np.float32, np.float64):
+        for n_left, batch, shape in [(1, 5, (9, 6)), (3, 1, (8, 8)), (4, 3, (12, 17))]:
+            say("overlap_wise batches", np.dtype(dtype).name, n_left, batch, shape)
+            left = ints(rng, (n_left,) + shape, dtype)
+            right = ints(rng, (n_left * batch,) + shape, dtype)
+            exp = oracle.n_to_mn(left, right)
+            got = xc.run("overlap_wise", left, right, n_left * batch, n_left=n_left, n_right=batch)
+            check(got, exp, True, f"overlap_wise {n_left}x{batch}")
+
+
+N_TO_MN_CASES = [
+    {},
+    dict(shifts_per_thread_right_matrix=4, right_matrices_per_thread=4, left_rows_per_iteration=4),
+    dict(shifts_per_thread_right_matrix=2, right_matrices_per_thread=1),
+    dict(rows_per_thread=8, distribution_type="rectangle"),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kw", N_TO_MN_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_n_to_mn_one_launch(oracle, dtype, kw):
+    """multimat_right_grouped with n_left > 1 takes the right matrices de-interleaved (left l
+    owns [l*m, (l+1)*m), as the reference's n_to_mn classes arrange them, n_to_mn.hpp:165-172);
+    the oracle works in file order, so the test interleaves around it with the reference's
+    index map (matrix.hpp:614-618)."""
+    xc = load_package()
+    rng = np.random.default_rng(400)
+    for n, m, shape in [(2, 3, (8, 8)), (3, 5, (20, 13)), (8, 4, (32, 32))]:
+        say("n_to_mn", kw, np.dtype(dtype).name, n, m, shape)
+        left = ints(rng, (n,) + shape, dtype)
+        right_file = ints(rng, (n * m,) + shape, dtype)
+        slot = [oracle.interleave_index(i, n * m, n) for i in range(n * m)]
+        right_dev = np.empty_like(right_file)
+        for i, s in enumerate(slot):
+            right_dev[s] = right_file[i]
+        exp_file = oracle.n_to_mn(left, right_file)
+        got_dev = xc.run("multimat_right_grouped", left, right_dev, n * m, n_left=n, n_right=m, params=xc.make_params(**kw))
+        got_file = np.stack([got_dev[slot[i]] for i in range(n * m)])
+        check(got_file, exp_file, True, f"n_to_mn {n}x{m} {shape}")
+
+
+N_TO_M_CASES = [
+    ("multimat_both", {}),
+    ("multimat_both", dict(left_matrices_per_thread=2, right_matrices_per_thread=2, rows_per_thread=10, distribution_type="triangle")),
+    ("multimat_both", dict(left_matrices_per_thread=8, right_matrices_per_thread=8, rows_per_thread=3, distribution_type="rectangle")),
+    ("multimat_both", dict(left_matrices_per_thread=1, right_matrices_per_thread=1, distribution_type="none")),
+    ("multimat_both_grouped", {}),
+    ("multimat_both_grouped", dict(shifts_per_thread_right_matrix=2, left_matrices_per_thread=2, right_matrices_per_thread=2, left_rows_per_iteration=2)),
+    ("multimat_both_grouped", dict(shifts_per_thread_right_matrix=4, left_matrices_per_thread=4, right_matrices_per_thread=4)),
+    ("multimat_both_grouped", dict(rows_per_thread=5)),
+]
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("family,kw", N_TO_M_CASES, ids=lambda v: str(v).replace(" ", ""))
+def test_n_to_m(oracle, dtype, family, kw):
+    xc = load_package()
+    rng = np.random.default_rng(500)
+    for n_left, n_right, shape in [(1, 1, (7, 7)), (2, 3, (16, 16)), (5, 9, (24, 31)), (16, 11, (32, 32))]:
+        say("n_to_m", family, kw, np.dtype(dtype).name, n_left, n_right, shape)
+        left = ints(rng, (n_left,) + shape, dtype)
+        right = ints(rng, (n_right,) + shape, dtype)
+        exp = oracle.n_to_m(left, right)
+        got = xc.run(family, left, right, n_left * n_right, n_left=n_left, n_right=n_right, params=xc.make_params(**kw))
+        check(got, exp, True, f"{family} {kw} {n_left}x{n_right} {shape} int")
+        left = rng.standard_normal((n_left,) + shape).astype(dtype)
+        right = rng.standard_normal((n_right,) + shape).astype(dtype)
+        exp = oracle.n_to_m(left, right, threads=4)
+        got = xc.run(family, left, right, n_left * n_right, n_left=n_left, n_right=n_right, params=xc.make_params(**kw))
+        check(got, exp, False, f"{family} {kw} {n_left}x{n_right} {shape} real")
+
+
+def test_every_tile_specialisation(oracle):
+    """Forces each lane layout / register tile through the geometry fields and checks it on
+    shapes that do not divide the tiles."""
+    xc = load_package()
+    rng = np.random.default_rng(600)
+    layouts = [dict(lanes_x=8, lanes_y=8), dict(lanes_x=4, lanes_y=4), dict(lanes_x=2, lanes_y=2), dict(lanes_x=1, lanes_y=1)]
+    for dtype in (np.float32, np.float64):
+        for lay in layouts:
+            for xs in (4, 8):
+                for n_left, n_right, shape in [(3, 5, (19, 23)), (9, 17, (40, 36))]:
+                    kw = dict(lay, x_shifts_per_thread=xs)
+                    left = ints(rng, (n_left,) + shape, dtype)
+                    right = ints(rng, (n_right,) + shape, dtype)
+                    try:
+                        got = xc.run("multimat_both_grouped", left, right, n_left * n_right, n_left=n_left, n_right=n_right,
+                                     params=xc.make_params(**kw))
+                    except xc.XcorrError as e:
+                        assert e.code == 3, e  # no such specialisation compiled
+                        continue
+                    say("tile", np.dtype(dtype).name, kw, xc.last_launch()["kernel"], n_left, n_right, shape)
+                    check(got, oracle.n_to_m(left, right), True, f"tile {kw} {shape}")
+
+
+def test_launch_record_and_errors():
+    xc = load_package()
+    rng = np.random.default_rng(700)
+    left = ints(rng, (32, 32), np.float32)
+    xc.run("grouped_overlap", left, left, 1, params=xc.make_params(shifts_per_thread=8))
+    rec = xc.last_launch()
+    say(rec)
+    assert rec["kernel"].startswith("grouped_overlap/")
+    assert rec["y_shifts_per_thread"] == 8 and rec["block"][0] % 64 == 0 and rec["grid"][0] >= 1
+    with pytest.raises(xc.XcorrError, match="Too many shifts per thread"):
+        xc.run("grouped_overlap", left, left, 1, params=xc.make_params(shifts_per_thread=9))
+    with pytest.raises(xc.XcorrError, match="Too many warps"):
+        xc.run("split_row", left, left, 1, params=xc.make_params(warps_per_thread_block=64))
+    info = xc.device_info()
+    say(info.name, info.arch, info.compute_units, info.clock_khz, info.fp32_vector_peak_tflops)
+    assert b"gfx950" in info.arch
