@@ -76,7 +76,8 @@ typedef struct xcorr_params {
     unsigned x_shifts_per_thread;            /* adjacent x shifts one lane accumulates: 4 or 8 */
     unsigned lanes_x;                        /* lanes of a wavefront laid along x shifts (power of two) */
     unsigned lanes_y;                        /* lanes laid along y shifts; the rest are laid over matrices */
-    unsigned reserved[3];
+    unsigned specialisation;                 /* 1-based index into the compiled tile list of the dtype (tuning sweeps) */
+    unsigned reserved[2];
 } xcorr_params;
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the

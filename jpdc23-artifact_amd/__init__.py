@@ -43,7 +43,8 @@ class Params(ctypes.Structure):
         ("x_shifts_per_thread", ctypes.c_uint),
         ("lanes_x", ctypes.c_uint),
         ("lanes_y", ctypes.c_uint),
-        ("reserved", ctypes.c_uint * 3),
+        ("specialisation", ctypes.c_uint),
+        ("reserved", ctypes.c_uint * 2),
     ]
 
 

@@ -20,8 +20,8 @@
 //     LDS, zero padded, so the inner loop has no bounds checks;
 //   * per left row and K right columns a lane reads one B+K-1 wide left window and
 //     one new right row of K values; the A right rows it needs are kept in a
-//     register ring that rotates by one row per step (the y loop is unrolled A times
-//     so every ring index is static). That is NV*NU*A*B*K FMAs for
+//     register ring that rotates by one row per step (the y loop is unrolled so every
+//     ring index is static), and every LDS read is issued one step ahead of its use. That is NV*NU*A*B*K FMAs for
 //     NV*ceil((B+K-1)/v) + NU*ceil(K/v) 128-bit LDS reads (v = 16 / sizeof(T));
 //   * the reduction over left rows can be split into chunks (work items) whose
 //     partial sums are added with hardware float atomics, which is what fills 256
@@ -59,20 +59,25 @@ struct EngineCfg {
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
     static constexpr int NWAVES = WX * WY, NT = 64 * NWAVES;
+    static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
     static constexpr int VWIN = B + K - 1;
     static constexpr int VWIN_VECS = (VWIN + VK - 1) / VK;
     static constexpr int KVECS = K / VK;
     static constexpr int NVB = LV * NV, NUB = LU * NU; // matrices per block
     // LDS geometry (elements)
     static constexpr int PV = TXB - B + KBX - K + VWIN_VECS * VK;
-    static constexpr int VBAND = RL * PV;
+    // Band sizes are padded to an odd number of 128-bit pieces: lanes laid over matrices read
+    // the same row and column of different bands in one instruction, and an odd stride puts
+    // eight such reads on eight different groups of four LDS banks.
+    static constexpr int odd_pieces(int n) { return ((n / VK) % 2) ? n : n + VK; }
+    static constexpr int VBAND = odd_pieces((RL + 1) * PV); // one spare row: the last step prefetches past the stage
     static constexpr int RU = RL + TYB - 1;
     static constexpr int PU = KBX + VK;
-    static constexpr int UBAND = RU * PU;
+    static constexpr int UBAND = odd_pieces((RU + 1) * PU);
     static constexpr int LDS_ELEMS = NVB * VBAND + NUB * UBAND;
     static constexpr int LDS_BYTES = LDS_ELEMS * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
-    static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % A == 0, "tile alignment");
+    static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -97,6 +102,99 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
     lo = syb > 0 ? syb : 0;
     int h = syb + C::TYB - 1 + H;
     hi = h < H ? h : H;
+}
+
+// Inner loops of one stage for one lane: for every K-column chunk kc in [kc_lo, kc_hi) sweep
+// the groups of G staged left rows jj in [jj_lo, jj_hi).
+//
+// Register plan per lane: NV*NU*A*B accumulators, a ring of G = A+1 right rows (row j in
+// slot j mod G, so the row of the next step is fetched while the current step still uses
+// all A of its rows) and ONE left window that is refilled in place: the FMAs of a step walk
+// the window element by element (anti-diagonals b + k = e of the B x K product grid), and
+// as soon as the last element of a 128-bit piece has been consumed the same piece of the
+// next row is requested. Every LDS read is thus in flight for at least half a step of FMAs
+// before its first use, without a second window buffer (which would push the tile past
+// 128 VGPRs and below four wavefronts per SIMD).
+template <class C>
+__device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
+                                              typename C::value_type (&acc)[C::NV][C::NU][C::A][C::B], int kc_lo,
+                                              int kc_hi, int jj_lo, int jj_hi) {
+    using T = typename C::value_type;
+    using vec = typename vec128<T>::type;
+    constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK, G = C::G;
+    constexpr int VW = C::VWIN_VECS * VK;
+    for (int kc = kc_lo; kc < kc_hi; ++kc) {
+        const T *vp = Vs_lane + kc * K + jj_lo * G * C::PV;
+        const T *up = Us_lane + kc * K + jj_lo * G * C::PU;
+        T ring[NU][G][K];
+        T vw[NV][VW];
+        // rows -(A-1) .. 0 of the right band, window of left row 0
+#pragma unroll
+        for (int n = 0; n < NU; ++n)
+#pragma unroll
+            for (int a = A - 1; a >= 0; --a)
+#pragma unroll
+                for (int q = 0; q < C::KVECS; ++q) {
+                    vec r = *reinterpret_cast<const vec *>(up + n * C::UBAND - a * C::PU + q * VK);
+#pragma unroll
+                    for (int e = 0; e < VK; ++e) ring[n][(G - a) % G][q * VK + e] = r[e];
+                }
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+            for (int q = 0; q < C::VWIN_VECS; ++q) {
+                vec r = *reinterpret_cast<const vec *>(vp + i * C::VBAND + q * VK);
+#pragma unroll
+                for (int e = 0; e < VK; ++e) vw[i][q * VK + e] = r[e];
+            }
+#pragma unroll 1
+        for (int jj = jj_lo; jj < jj_hi; ++jj) {
+#pragma unroll
+            for (int s = 0; s < G; ++s) {
+                // right row s+1 (at s = G-1: the first row of the next group, or the spare
+                // row the bands keep at their end)
+#pragma unroll
+                for (int n = 0; n < NU; ++n)
+#pragma unroll
+                    for (int q = 0; q < C::KVECS; ++q) {
+                        vec r = *reinterpret_cast<const vec *>(up + n * C::UBAND + (s + 1) * C::PU + q * VK);
+#pragma unroll
+                        for (int e = 0; e < VK; ++e) ring[n][(s + 1) % G][q * VK + e] = r[e];
+                    }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int e = 0; e < C::VWIN; ++e) {
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        const int b = e - k;
+                        if (b < 0 || b >= B) continue;
+#pragma unroll
+                        for (int i = 0; i < NV; ++i)
+#pragma unroll
+                            for (int n = 0; n < NU; ++n)
+#pragma unroll
+                                for (int a = 0; a < A; ++a) acc[i][n][a][b] += vw[i][e] * ring[n][(s - a + G) % G][k];
+                    }
+                    if (e % VK == VK - 1 || e == C::VWIN - 1) {
+                        // this 128-bit piece of the window is consumed: refill it from the next row
+                        // (the scheduling fences keep the compiler from sinking the read down to
+                        // its first use in the next step, which would expose the LDS latency)
+                        const int q = e / VK;
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int i = 0; i < NV; ++i) {
+                            vec r = *reinterpret_cast<const vec *>(vp + i * C::VBAND + (s + 1) * C::PV + q * VK);
+#pragma unroll
+                            for (int x = 0; x < VK; ++x) vw[i][q * VK + x] = r[x];
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            vp += G * C::PV;
+            up += G * C::PU;
+        }
+    }
 }
 
 template <class C>
@@ -175,10 +273,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wx = wave % C::WX, wy = wave / C::WX;
+    // x fastest, y slowest: the eight lanes an LDS access serves together then differ in what
+    // selects the LEFT address (x, left matrix) and share the right-row address, or differ in
+    // the right matrix only; rows that are a multiple of A apart (different y) would always
+    // fall on the same banks
     const int lx = lane % C::LX;
-    const int ly = (lane / C::LX) % C::LY;
-    const int lv = (lane / (C::LX * C::LY)) % C::LV;
-    const int lu = lane / (C::LX * C::LY * C::LV);
+    const int lv = (lane / C::LX) % C::LV;
+    const int lu = (lane / (C::LX * C::LV)) % C::LU;
+    const int ly = lane / (C::LX * C::LV * C::LU);
     const int sxw = sxb + wx * C::TXW; // first x shift of the wavefront tile
     const int syw = syb + wy * C::TYW;
     const T *Vs_lane = Vs + lv * NV * C::VBAND + wx * C::TXW + lx * B;
@@ -198,15 +300,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const size_t HW = (size_t)W * H;
 
     for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
-        // groups of A left rows of this stage that can overlap this wavefront's y shifts
-        int jj_lo = 0, jj_hi = C::RL / A;
+        // groups of G left rows of this stage that can overlap this wavefront's y shifts
+        int jj_lo = 0, jj_hi = C::RL / C::G;
         {
             // rows yl in [syw, syw + TYW - 1 + H - 1] and yl < chi
             int first = syw - yl0;                     // first useful row index j
             int last = syw + C::TYW + H - 2 - yl0;     // last useful row index j
             if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
-            if (first > 0) jj_lo = first / A;
-            int h = last < 0 ? 0 : last / A + 1;
+            if (first > 0) jj_lo = first / C::G;
+            int h = last < 0 ? 0 : last / C::G + 1;
             if (h < jj_hi) jj_hi = h;
         }
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
@@ -214,34 +316,36 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             // ---- stage the left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col ----
             {
                 const int xbase = x0 + sxb;
-                constexpr int TOT = C::NVB * C::VBAND;
-#pragma unroll 4
+                constexpr int TOT = C::NVB * (C::RL + 1) * C::PV;
+#pragma unroll
                 for (int idx = tid; idx < TOT; idx += C::NT) {
                     int col = idx % C::PV;
                     int t = idx / C::PV;
-                    int row = t % C::RL;
-                    int band = t / C::RL;
+                    int row = t % (C::RL + 1);
+                    int band = t / (C::RL + 1);
                     int v = v_first + band, yl = yl0 + row, xl = xbase + col;
+                    int dst = band * C::VBAND + row * C::PV + col;
                     T val = T(0);
-                    if (v < g.nV && yl < chi && (unsigned)xl < (unsigned)W) val = g.V[(size_t)v * HW + (size_t)yl * W + xl];
-                    Vs[idx] = val;
+                    if (v < g.nV && row < C::RL && yl < chi && (unsigned)xl < (unsigned)W) val = g.V[(size_t)v * HW + (size_t)yl * W + xl];
+                    Vs[dst] = val;
                 }
             }
             // ---- stage the right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col ----
             {
                 const int yr0 = yl0 - syb - C::TYB + 1;
-                constexpr int TOT = C::NUB * C::UBAND;
-#pragma unroll 4
+                constexpr int TOT = C::NUB * (C::RU + 1) * C::PU;
+#pragma unroll
                 for (int idx = tid; idx < TOT; idx += C::NT) {
                     int col = idx % C::PU;
                     int t = idx / C::PU;
-                    int row = t % C::RU;
-                    int band = t / C::RU;
+                    int row = t % (C::RU + 1);
+                    int band = t / (C::RU + 1);
                     int u = u_first + band, yr = yr0 + row, xr = x0 + col;
+                    int dst = band * C::UBAND + row * C::PU + col;
                     T val = T(0);
                     if (u < u_limit && col < C::KBX && (unsigned)yr < (unsigned)H && xr < W)
                         val = g.U[(size_t)u * HW + (size_t)yr * W + xr];
-                    Us[idx] = val;
+                    Us[dst] = val;
                 }
             }
             __syncthreads();
@@ -259,58 +363,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             }
             if (jj_lo >= jj_hi) continue;
 
-            for (int kc = kc_lo; kc < kc_hi; ++kc) {
-                const T *vp = Vs_lane + kc * K + jj_lo * A * C::PV;
-                const T *up = Us_lane + kc * K + jj_lo * A * C::PU;
-                // ring[n][s] holds right row (j - a) of matrix n in slot s = (j - a) mod A
-                T ring[NU][A][K];
-#pragma unroll
-                for (int n = 0; n < NU; ++n)
-#pragma unroll
-                    for (int a = 1; a < A; ++a)
-#pragma unroll
-                        for (int q = 0; q < C::KVECS; ++q) {
-                            vec r = *reinterpret_cast<const vec *>(up + n * C::UBAND - a * C::PU + q * VK);
-#pragma unroll
-                            for (int e = 0; e < VK; ++e) ring[n][(A - a) % A][q * VK + e] = r[e];
-                        }
-#pragma unroll 1
-                for (int jj = jj_lo; jj < jj_hi; ++jj) {
-#pragma unroll
-                    for (int s = 0; s < A; ++s) {
-#pragma unroll
-                        for (int n = 0; n < NU; ++n)
-#pragma unroll
-                            for (int q = 0; q < C::KVECS; ++q) {
-                                vec r = *reinterpret_cast<const vec *>(up + n * C::UBAND + s * C::PU + q * VK);
-#pragma unroll
-                                for (int e = 0; e < VK; ++e) ring[n][s][q * VK + e] = r[e];
-                            }
-                        T vw[NV][C::VWIN_VECS * VK];
-#pragma unroll
-                        for (int i = 0; i < NV; ++i)
-#pragma unroll
-                            for (int q = 0; q < C::VWIN_VECS; ++q) {
-                                vec r = *reinterpret_cast<const vec *>(vp + i * C::VBAND + s * C::PV + q * VK);
-#pragma unroll
-                                for (int e = 0; e < VK; ++e) vw[i][q * VK + e] = r[e];
-                            }
-#pragma unroll
-                        for (int k = 0; k < K; ++k)
-#pragma unroll
-                            for (int i = 0; i < NV; ++i)
-#pragma unroll
-                                for (int n = 0; n < NU; ++n)
-#pragma unroll
-                                    for (int a = 0; a < A; ++a)
-#pragma unroll
-                                        for (int b = 0; b < B; ++b)
-                                            acc[i][n][a][b] += vw[i][b + k] * ring[n][(s - a + A) % A][k];
-                    }
-                    vp += A * C::PV;
-                    up += A * C::PU;
-                }
-            }
+            compute_stage<C>(Vs_lane, Us_lane, acc, kc_lo, kc_hi, jj_lo, jj_hi);
         }
     }
 

@@ -1,25 +1,27 @@
 // fp64 specialisations of the sliding-window engine. The reference has no fp64 GPU
 // path (its double instantiations are commented out, e.g.
 // naive_shuffle_multirow_both.cu:701-710); these use v_fma_f64 with K = 2 columns per
-// 128-bit LDS access.
+// 128-bit LDS access. An 8x8 tile of doubles needs ~190 VGPRs (two wavefronts per SIMD).
 #include "engine_registry.hpp"
 
 namespace xcorr {
 
-//                          T       A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB
-using R_1x1 = EngineCfg<double, 1, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 8, 16, 4>;
-using R_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 1, 1, 8, 16, 4>;
-using G_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 16, 16, 2>;
-using G_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 16, 16, 2>;
-using G_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 1, 1, 16, 16, 2>;
-using G_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 1, 1, 16, 8, 2>;
-using G_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 16, 16, 2>;
-using G_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 1, 1, 16, 16, 2>;
+//                           T       A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB
+using R_1x1 = EngineCfg<double, 1, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
+using R_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
+using G_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 18, 16, 2>;
+using G_88_w1 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 18, 16, 2>;
+using G_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 2, 2, 20, 16, 4>;
+using G_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 2, 2, 18, 8, 2>;
+using G_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 2, 2, 9, 4, 2>;
+using G_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 2, 2, 9, 8, 2>;
+using G_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 2, 2, 18, 8, 2>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
     make_spec<R_2x2>("f64_a1b4_l2r2"),
     make_spec<G_88>("f64_a8b8"),
+    make_spec<G_88_w1>("f64_a8b8_w1"),
     make_spec<G_44>("f64_a4b4"),
     make_spec<G_88_u4>("f64_a8b8_lr4"),
     make_spec<G_88_u16>("f64_a8b8_lr16"),

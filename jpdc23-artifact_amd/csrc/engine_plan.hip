@@ -25,25 +25,33 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)); }
 
-// Relative cost of running the request on a specialisation: work issued for partial
-// overlaps at tile edges, lanes idling over matrices that do not exist, and LDS read
-// time when a tile has too little register reuse. Hints scale the cost so the nearest
-// specialisation wins without excluding the others.
+// Relative cost of running the request on a specialisation, calibrated on MI355X sweeps:
+//   * work issued for partial overlaps at tile edges. Wavefronts skip what cannot overlap
+//     their own tile, but the waves of a block meet at a barrier after every staged band,
+//     so both the wavefront tile and the block tile count;
+//   * lanes idling over matrices that do not exist;
+//   * issue slots lost to LDS reads: a read plus the wait that guards it displace about nine
+//     fp32 FMA slots (half as many fp64 ones) of the wavefront that issues them;
+//   * lanes laid over matrices stage many small bands and write one matrix per lane.
+// Hints scale the cost so the nearest specialisation wins without excluding the others.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
-    double waste_x = (double)(rq.W + s.TXW()) / rq.W;
-    double waste_y = (double)(rq.H + s.TYW()) / rq.H;
+    // geometric mean of the wavefront-tile and block-tile overheads
+    double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
+    double waste_y = std::sqrt((double)(rq.H + s.TYW()) * (rq.H + s.TYB())) / rq.H;
     int nu = rq.group_m > 0 ? rq.group_m : rq.nU;
     double util_v = (double)rq.nV / ((double)ceil_div(rq.nV, s.NVB()) * s.NVB());
     double util_u = (double)nu / ((double)ceil_div(nu, s.NUB()) * s.NUB());
     int vk = 16 / s.elem_bytes;
     double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
     double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
-    double lds = 8.0 * reads / fmas * 1.15; // LDS cycles per VALU cycle with four SIMDs sharing one LDS
-    double cost = waste_x * waste_y / (util_v * util_u) * (lds > 1.0 ? lds : 1.0);
-    // very small grids cannot fill the device: prefer narrower tiles then
-    if (rq.y_shifts > 1) cost *= 1.0 + 0.25 * log2_ratio(s.A, rq.y_shifts);
-    if (rq.left_mats) cost *= 1.0 + 0.25 * log2_ratio(s.NV, rq.left_mats);
-    if (rq.right_mats) cost *= 1.0 + 0.25 * log2_ratio(s.NU, rq.right_mats);
+    double issue = 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
+    double cost = waste_x * waste_y / (util_v * util_u) * issue;
+    if (s.LV * s.LU > 1) cost *= 2.0;
+    if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
+    if (s.WX * s.WY < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
+    if (rq.y_shifts > 1) cost *= 1.0 + 3.0 * log2_ratio(s.A, rq.y_shifts);
+    if (rq.left_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NV, rq.left_mats);
+    if (rq.right_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NU, rq.right_mats);
     if (rq.waves) cost *= 1.0 + 0.05 * log2_ratio(s.WX * s.WY, rq.waves);
     return cost;
 }
@@ -53,7 +61,15 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     const EngineSpec *specs = rq.elem_bytes == 4 ? engine_specs_f32(&count) : engine_specs_f64(&count);
     const EngineSpec *best = nullptr;
     double best_cost = 0;
-    for (int i = 0; i < count; ++i) {
+    if (rq.spec_index > 0) {
+        if ((int)rq.spec_index > count)
+            return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %u does not exist (%d compiled)", rq.family, rq.spec_index, count);
+        const EngineSpec &s = specs[rq.spec_index - 1];
+        if (rq.group_m > 0 && s.NVB() != 1)
+            return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %s cannot pair one left matrix with a group", rq.family, s.name);
+        best = &s;
+    }
+    for (int i = 0; i < count && rq.spec_index == 0; ++i) {
         const EngineSpec &s = specs[i];
         if ((rq.y_shifts == 1) != (s.A == 1)) continue; // one-output-row families vs grouped families
         if (rq.group_m > 0 && s.NVB() != 1) continue;
@@ -87,9 +103,15 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         plan.atomic = 1;
         plan.zero_fill = false;
     } else {
-        if (rc <= 0 && rq.may_split) {
-            const long target = 16L * device_cus();
+        // lanes laid over matrices write one result matrix per lane: their atomics would not
+        // coalesce, so such tiles are never split by the planner itself
+        const bool split_ok = rq.may_split && best->LV * best->LU == 1;
+        if (rc <= 0 && split_ok) {
+            const long target = 32L * device_cus();
             long chunks_wanted = (target + tiles - 1) / tiles;
+            // a work item should span at least two staged bands of left rows
+            long most = rq.H / (2 * best->RL);
+            if (chunks_wanted > most) chunks_wanted = most;
             if (chunks_wanted > 1) {
                 rc = ceil_div(rq.H, (int)chunks_wanted);
                 rc = ceil_div(rc, best->RL) * best->RL;

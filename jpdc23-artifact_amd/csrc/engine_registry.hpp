@@ -71,6 +71,7 @@ struct EngineRequest {
     int group_m;          // see EngineArgs
     // hints (0 = none). y_shifts == 1 selects the one-output-row-per-lane specialisations.
     unsigned y_shifts, x_shifts, left_mats, right_mats, lanes_x, lanes_y, waves;
+    unsigned spec_index;      // 1-based: use exactly this entry of the specialisation table
     unsigned rows_per_worker; // 0 = planner decides
     unsigned dist;            // XCORR_DIST_*
     bool caller_zeroes;       // true: split-row contract, output arrives zeroed, always accumulate atomically

@@ -159,6 +159,7 @@ EngineRequest base_request(const char *family, int elem_bytes, const void *left,
     rq.x_shifts = p.x_shifts_per_thread;
     rq.lanes_x = p.lanes_x;
     rq.lanes_y = p.lanes_y;
+    rq.spec_index = p.specialisation;
     rq.waves = waves_from_warps(p.warps_per_thread_block);
     rq.dist = p.distribution_type;
     return rq;
@@ -207,7 +208,6 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     if ((rc = check_dist(p.distribution_type))) return rc;
     EngineRequest rq = base_request("grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = p.shifts_per_thread == 1 ? 2 : p.shifts_per_thread; // 0 = planner's choice among the grouped tiles
-    if (rq.y_shifts == 0) rq.y_shifts = 0;
     rq.rows_per_worker = p.rows_per_thread;
     rq.may_split = true;
     return run_engine(rq, as_stream(stream));
