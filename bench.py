@@ -19,8 +19,12 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 from __graft_entry__ import load_oracle, load_package  # noqa: E402
 
-# MI355X published vector peaks (TFLOP/s); fp32 assumes packed FMA
+# MI355X published vector peaks (TFLOP/s)
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
+# by the library's copy kernel (figures and commands: profiles/engine_f32_a8b8_one_to_one_1024.md).
+# Only the default workload with default parameters has been measured.
+MEASURED_TRAFFIC_BYTES = {"C2": 0.812e9 + 1.495e9}
 
 
 def cpu_baseline(oracle, cfg, left, right, budget_s=15.0):
@@ -70,6 +74,9 @@ def main():
     ap.add_argument("--family", default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--params", default="{}", help="JSON object of xcorr_params fields")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch the library's plain copy kernel on 256 MiB so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "readings of the same run can be scaled to bytes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every output element is an independent reduction; "
@@ -105,6 +112,19 @@ def main():
         if zero_first:
             d_out.zero()
         xc.launch(family, d_left, d_right, d_out, cols, rows, n_left, n_right, dtype, params)
+
+    if args.calibrate_copy:
+        import ctypes
+
+        nbytes = 256 * 1024 * 1024
+        src, dst = xc.DeviceBuffer(nbytes), xc.DeviceBuffer(nbytes)
+        src.zero()
+        for _ in range(3):  # each launch reads 256 MiB and writes 256 MiB
+            code = xc.lib().xcorr_copy_kernel(dst.ptr, src.ptr, ctypes.c_size_t(nbytes), None)
+            assert code == 0, xc.lib().xcorr_last_error()
+        xc.sync()
+        src.free()
+        dst.free()
 
     for _ in range(args.warmup):
         step()
@@ -157,10 +177,11 @@ def main():
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(achieved_tflops / peak, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.config) if (args.family is None and args.params == "{}") else None,
+            "algorithmic_bytes": workloads.algorithmic_bytes(cfg),
             "kernel_ms": round(kernel_ms, 4),
-            "note": "vector-FMA roofline (MFMA is not used); peak is the published packed-FP32 figure, "
-                    "plain v_fma_f32 (the only form this build emits) tops out at 0.5 of it" if dtype == np.float32 else
+            "note": "vector-FMA roofline (MFMA is not used); the kernel issues plain v_fmac_f32, which measures "
+                    "0.97 of this peak in a register-only loop on MI355X" if dtype == np.float32 else
                     "vector-FMA roofline, v_fma_f64",
         },
     }

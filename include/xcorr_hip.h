@@ -124,6 +124,9 @@ const char *xcorr_version(void);
 int xcorr_malloc(void **dev_ptr, size_t bytes);
 int xcorr_free(void *dev_ptr);
 int xcorr_memset_async(void *dev_ptr, int value, size_t bytes, void *stream);
+/* plain device-to-device copy KERNEL (16 bytes per lane), no reference counterpart: a launch of
+ * known read and write size against which memory-traffic counters are calibrated */
+int xcorr_copy_kernel(void *dev_dst, const void *dev_src, size_t bytes, void *stream);
 int xcorr_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes);
 int xcorr_memcpy_d2h(void *host_dst, const void *dev_src, size_t bytes);
 int xcorr_memcpy_h2d_async(void *dev_dst, const void *host_src, size_t bytes, void *stream);

@@ -8,6 +8,12 @@ using namespace xcorr;
 
 static hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
+__global__ void xcorr_plain_copy_kernel(uint4 *__restrict__ dst, const uint4 *__restrict__ src, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
+
 extern "C" {
 
 // ------------------------------------------------------------------ status
@@ -55,6 +61,18 @@ int xcorr_free(void *dev_ptr) {
 }
 int xcorr_memset_async(void *dev_ptr, int value, size_t bytes, void *stream) {
     XCORR_HIP(hipMemsetAsync(dev_ptr, value, bytes, as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_copy_kernel(void *dev_dst, const void *dev_src, size_t bytes, void *stream) {
+    if (!dev_dst || !dev_src) return fail(XCORR_ERR_INVALID_ARGUMENT, "null device pointer");
+    if (bytes % 16 != 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "copy size %zu is not a multiple of 16 bytes", bytes);
+    if (bytes == 0) return XCORR_OK;
+    size_t n = bytes / 16;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    xcorr_plain_copy_kernel<<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(static_cast<uint4 *>(dev_dst),
+                                                                                       static_cast<const uint4 *>(dev_src), n);
+    XCORR_HIP(hipGetLastError());
     return XCORR_OK;
 }
 int xcorr_memcpy_h2d(void *dev_dst, const void *host_src, size_t bytes) {

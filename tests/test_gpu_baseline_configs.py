@@ -1,0 +1,157 @@
+"""The five benchmark configurations at their full sizes, through the C ABI.
+
+The CPU oracle needs minutes to hours at these sizes, so parity is established through
+properties that do not depend on size:
+  * integer-valued inputs: every product and partial sum is an exactly representable integer,
+    so the result is independent of the summation order and must equal, bit for bit, the
+    correlation computed with double-precision FFTs and rounded to the nearest integer (the FFT
+    identity itself is checked against the oracle at a small size first);
+  * real-valued seeded inputs: relative Frobenius error against the double-precision FFT
+    result at most 1e-5 (fp32) / 1e-12 (fp64), the tolerances of the build's brief; the max
+    element error is printed;
+  * the all-ones closed form at the largest size;
+  * a band of central output rows of the largest configuration against the oracle itself.
+"""
+import numpy as np
+import pytest
+
+from conftest import load_package
+
+pytestmark = pytest.mark.gpu
+
+
+def fft_xcorr(left, right):
+    """Full cross-correlation of two equally sized matrices in double precision via FFT."""
+    rows, cols = left.shape
+    shape = (2 * rows - 1, 2 * cols - 1)
+    f = np.fft.rfft2(left.astype(np.float64), shape) * np.fft.rfft2(right.astype(np.float64)[::-1, ::-1], shape)
+    return np.fft.irfft2(f, shape)
+
+
+def fft_reference(cfg, left, right, workloads):
+    out = []
+    for l, r, _ in workloads.pair_list(cfg):
+        out.append(fft_xcorr(left[l], right[r]))
+    return np.stack(out)
+
+
+def device_order(cfg, right):
+    """n_to_mn inputs are generated in file order; the one-launch entry point takes the right
+    matrices grouped per left matrix."""
+    if cfg["mode"] != "n_to_mn":
+        return right, None
+    n = cfg["n_left"]
+    m = cfg["n_right"] // n
+    slot = np.array([(i % n) * m + i // n for i in range(n * m)])
+    grouped = np.empty_like(right)
+    grouped[slot] = right
+    return grouped, slot
+
+
+def run_config(xc, cfg, left, right, family=None, params=None):
+    n_left = cfg["n_left"]
+    n_right = cfg["n_right"] // n_left if cfg["mode"] == "n_to_mn" else cfg["n_right"]
+    right_dev, slot = device_order(cfg, right)
+    pairs = cfg["n_left"] * cfg["n_right"] if cfg["mode"] == "n_to_m" else cfg["n_right"]
+    got = xc.run(family or cfg["family"], left, right_dev, pairs, n_left=n_left, n_right=n_right,
+                 params=xc.make_params(**(params if params is not None else cfg.get("params", {}))))
+    return got if slot is None else got[slot]
+
+
+def test_fft_identity_matches_oracle(oracle):
+    rng = np.random.default_rng(0)
+    a = rng.integers(-5, 6, size=(9, 14)).astype(np.float64)
+    b = rng.integers(-5, 6, size=(9, 14)).astype(np.float64)
+    np.testing.assert_array_equal(np.rint(fft_xcorr(a, b)), oracle.cross_corr(a, b))
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_integer_inputs_bit_exact_at_full_size(name):
+    xc = load_package()
+    from jpdc23_artifact_amd import workloads
+
+    cfg = dict(workloads.CONFIGS[name])
+    left, right = workloads.generate(cfg, integer_valued=True)
+    print(name, cfg["mode"], left.shape, right.shape, flush=True)
+    got = run_config(xc, cfg, left, right)
+    exp = np.rint(fft_reference(cfg, left, right, workloads))
+    assert np.abs(exp).max() < 2 ** 24
+    print(name, xc.last_launch()["kernel"], "max |value|", np.abs(exp).max(), flush=True)
+    np.testing.assert_array_equal(got, exp.astype(got.dtype))
+
+
+@pytest.mark.parametrize("name,family", [
+    ("C1", None), ("C1", "grouped_overlap"), ("C1", "split_row"), ("C2", None), ("C2", "split_row"),
+    ("C3", None), ("C3", "multimat_right"), ("C4", None), ("C5", None), ("C5", "multimat_both"),
+])
+def test_seeded_inputs_within_tolerance_at_full_size(name, family):
+    xc = load_package()
+    from jpdc23_artifact_amd import workloads
+
+    cfg = dict(workloads.CONFIGS[name])
+    left, right = workloads.generate(cfg)
+    if family in ("multimat_right", "multimat_both", "split_row"):
+        params = dict(rows_per_thread=64, distribution_type="triangle")
+    else:
+        params = None if family is None else {}
+    got = run_config(xc, cfg, left, right, family=family, params=params)
+    exp = fft_reference(cfg, left, right, workloads)
+    err = np.linalg.norm(got.astype(np.float64).ravel() - exp.ravel()) / np.linalg.norm(exp.ravel())
+    max_abs = np.abs(got - exp).max()
+    tol = 1e-5 if cfg["dtype"] == "float32" else 1e-12
+    print(f"{name} {xc.last_launch()['kernel']}: rel_frobenius={err:.3e} max_abs={max_abs:.3e} max|ref|={np.abs(exp).max():.3e}", flush=True)
+    assert np.isfinite(got).all()
+    assert err <= tol
+
+
+def test_all_ones_closed_form_1024():
+    xc = load_package()
+    n = 1024
+    ones = np.ones((n, n), dtype=np.float32)
+    got = xc.run("grouped_overlap", ones, ones, 1)[0]
+    o = np.arange(2 * n - 1)
+    exp = np.outer(n - np.abs(o - (n - 1)), n - np.abs(o - (n - 1))).astype(np.float32)
+    np.testing.assert_array_equal(got, exp)
+
+
+def test_c2_band_against_oracle(oracle):
+    """Sixteen central output rows of the 1024x1024 pair against the oracle.
+
+    The reference's host loop adds ~10^6 positive products one by one in fp32; at the centre of
+    this configuration that loses about 1.2e-4 relative to the exact sum (the fp64-accumulating
+    variant of the same loop shows it). Two things are asserted:
+      * the default launch, which splits the reduction into chunks of a few dozen left rows and
+        therefore rounds less, is within 1e-5 of the exactly accumulated result;
+      * the same entry point asked not to split (rows_per_thread >= rows: one worker per tile,
+        every accumulator runs over the whole overlap like a thread of the reference's kernel
+        does) reproduces the fp32 host loop itself to 1e-5.
+    All three pairwise differences are printed with their max element error."""
+    xc = load_package()
+    from jpdc23_artifact_amd import workloads
+
+    cfg = dict(workloads.CONFIGS["C2"])
+    left, right = workloads.generate(cfg)
+    lo, hi = 1015, 1031
+    ref32 = oracle.cross_corr(left[0], right[0], threads=16, row_begin=lo, row_end=hi)[lo:hi]
+    ref64 = oracle.cross_corr(left[0], right[0], threads=16, row_begin=lo, row_end=hi, acc64=True)[lo:hi]
+    o64 = oracle.errors(ref32, ref64)
+    print(f"fp32 host loop vs fp64-accumulated: rel_frobenius={o64.rel_frobenius:.3e} max_abs={o64.max_abs:.3e}", flush=True)
+
+    got = xc.run("grouped_overlap", left, right, 1)[0]
+    rec = xc.last_launch()
+    e32 = oracle.errors(got[lo:hi], ref32)
+    e64 = oracle.errors(got[lo:hi], ref64)
+    print(f"default ({rec['kernel']}, {rec['rows_per_worker']} rows per worker) vs fp32 host loop: "
+          f"rel_frobenius={e32.rel_frobenius:.3e} max_abs={e32.max_abs:.3e} max_rel={e32.max_rel:.3e}", flush=True)
+    print(f"default vs fp64-accumulated: rel_frobenius={e64.rel_frobenius:.3e} max_abs={e64.max_abs:.3e}", flush=True)
+    assert e64.rel_frobenius <= 1e-5
+
+    got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(rows_per_thread=1024))[0]
+    rec = xc.last_launch()
+    assert rec["uses_atomics"] == 0
+    u32 = oracle.errors(got[lo:hi], ref32)
+    u64 = oracle.errors(got[lo:hi], ref64)
+    print(f"unsplit ({rec['kernel']}) vs fp32 host loop: rel_frobenius={u32.rel_frobenius:.3e} max_abs={u32.max_abs:.3e} "
+          f"max_rel={u32.max_rel:.3e}", flush=True)
+    print(f"unsplit vs fp64-accumulated: rel_frobenius={u64.rel_frobenius:.3e} max_abs={u64.max_abs:.3e}", flush=True)
+    assert u32.rel_frobenius <= 1e-5
