@@ -46,19 +46,26 @@ struct EngineArgs {
     int ntx, nty;       // number of block tiles in x and y
     int nworkers_y;     // number of (y tile, chunk) workers
     int nvg, nug;       // left / right matrix groups
+    int total_items;    // nvg * nug * nworkers_y * ntx
 };
 
+// IW_ > 1: the IW_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
+// matrices and split its left rows among themselves: each stages its own LDS bands, runs without
+// workgroup barriers, and the partial sums are added through LDS before the tile is written. This
+// divides the longest work item of a launch by IW_ without atomics, which is what small matrices
+// laid over lanes need: their central tiles would otherwise run long after the rest has finished.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
-          int RL_, int KBX_, int MINB_>
+          int RL_, int KBX_, int MINB_, int IW_ = 1>
 struct EngineCfg {
     using value_type = T;
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
-    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_;
+    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, IW = IW_;
     static constexpr int VK = 16 / (int)sizeof(T); // elements per 128-bit LDS access
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
-    static constexpr int NWAVES = WX * WY, NT = 64 * NWAVES;
+    static constexpr int NWAVES = WX * WY, NT = 64 * NWAVES * IW;
+    static constexpr int ITEM_THREADS = 64 * NWAVES; // threads that cooperate on one work item
     static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
     static constexpr int VWIN = B + K - 1;
     static constexpr int VWIN_VECS = (VWIN + VK - 1) / VK;
@@ -75,8 +82,12 @@ struct EngineCfg {
     static constexpr int PU = KBX + VK;
     static constexpr int UBAND = odd_pieces((RU + 1) * PU);
     static constexpr int LDS_ELEMS = NVB * VBAND + NUB * UBAND;
-    static constexpr int LDS_BYTES = LDS_ELEMS * (int)sizeof(T);
+    // in-block reduction: one output row of the tile per wavefront and pass, [owner][source][lane][RED_ROW]
+    static constexpr int RED_ROW = NV * NU * B;
+    static constexpr int RED_ELEMS = IW > 1 ? IW * IW * 64 * RED_ROW : 0;
+    static constexpr int LDS_BYTES = (LDS_ELEMS * IW > RED_ELEMS ? LDS_ELEMS * IW : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
+    static_assert(IW == 1 || (WX == 1 && WY == 1 && A % IW == 0), "row-splitting wavefronts share one wavefront tile");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
@@ -92,6 +103,44 @@ struct vec128<double> {
     typedef double type __attribute__((ext_vector_type(2)));
 };
 
+// Cycle accounting per phase of engine_kernel, compiled in with -DXCORR_ENGINE_PROFILE only (a
+// tuning aid: every wavefront adds the shader-clock cycles it spent per phase to a device-side
+// table that engine_profile_read() copies out and clears).
+enum EnginePhase { PH_SETUP, PH_WAIT_SIBLINGS, PH_STAGING, PH_WAIT_STAGED, PH_COMPUTE, PH_OUTPUT, PH_COUNT };
+#ifdef XCORR_ENGINE_PROFILE
+static __device__ unsigned long long engine_profile[PH_COUNT + 2]; // phases, wavefronts, first-to-last cycles
+struct PhaseClock {
+    long long t0, t, acc[PH_COUNT];
+    __device__ __forceinline__ PhaseClock() {
+        for (int i = 0; i < PH_COUNT; ++i) acc[i] = 0;
+        t0 = t = (long long)clock64();
+    }
+    __device__ __forceinline__ void lap(int phase) {
+        long long now = (long long)clock64();
+        acc[phase] += now - t;
+        t = now;
+    }
+    __device__ __forceinline__ void flush() {
+        if ((threadIdx.x & 63) == 0) {
+            for (int i = 0; i < PH_COUNT; ++i) atomicAdd(&engine_profile[i], (unsigned long long)acc[i]);
+            atomicAdd(&engine_profile[PH_COUNT], 1ull);
+            atomicAdd(&engine_profile[PH_COUNT + 1], (unsigned long long)(t - t0));
+        }
+    }
+};
+static inline hipError_t engine_profile_read(unsigned long long *out) {
+    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(engine_profile), sizeof(engine_profile));
+    if (e != hipSuccess) return e;
+    unsigned long long zero[PH_COUNT + 2] = {};
+    return hipMemcpyToSymbol(HIP_SYMBOL(engine_profile), zero, sizeof(zero));
+}
+#else
+struct PhaseClock {
+    __device__ __forceinline__ void lap(int) {}
+    __device__ __forceinline__ void flush() {}
+};
+#endif
+
 __device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 
@@ -102,6 +151,64 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
     lo = syb > 0 ? syb : 0;
     int h = syb + C::TYB - 1 + H;
     hi = h < H ? h : H;
+}
+
+// Orders the LDS writes of a stage before its reads (and the reads before the next stage's
+// writes) among the threads that share a work item: a workgroup barrier, or nothing but a
+// compiler fence when the item belongs to a single wavefront (the LDS serves the accesses of
+// one wavefront in program order).
+template <class C>
+__device__ __forceinline__ void item_sync() {
+    if (C::IW > 1)
+        __builtin_amdgcn_wave_barrier();
+    else
+        __syncthreads();
+}
+
+// Fills the LDS image of NB bands (ROWS rows of PITCH elements, BAND elements apart) from NB
+// matrices that are `mat_stride` elements apart in global memory. Image element (band, row, col)
+// is src[band][row0 + row][col0 + col] if band < nbands, row_lo <= row < row_hi and
+// col_lo <= col < col_hi, and zero otherwise (the caller passes ranges that keep the reads
+// inside the matrices). Every thread moves 128-bit pieces; the loads of up to eight pieces are
+// issued back to back before the first LDS write, so their latencies overlap.
+template <class C, int NB, int ROWS, int PITCH, int BAND>
+__device__ __forceinline__ void stage_bands(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride, int W,
+                                            int nbands, int row_lo, int row_hi, int row0, int col0, int col_lo, int col_hi, int tid) {
+    using T = typename C::value_type;
+    using vec = typename vec128<T>::type;
+    constexpr int VK = C::VK, PP = PITCH / VK, TOTP = NB * ROWS * PP;
+    constexpr int ITER = (TOTP + C::ITEM_THREADS - 1) / C::ITEM_THREADS;
+    constexpr int BATCH = ITER < 8 ? ITER : 8;
+    static_assert(PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
+#pragma unroll
+    for (int it0 = 0; it0 < ITER; it0 += BATCH) {
+        vec val[BATCH];
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            const int p = tid + (it0 + j) * C::ITEM_THREADS;
+            const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
+            vec v;
+#pragma unroll
+            for (int e = 0; e < VK; ++e) v[e] = T(0);
+            if (it0 + j < ITER && band < nbands && row >= row_lo && row < row_hi && col + VK > col_lo && col < col_hi) {
+                const T *q = src + (size_t)band * mat_stride + (size_t)(row0 + row) * W + (ptrdiff_t)(col0 + col);
+                if (col >= col_lo && col + VK <= col_hi) {
+                    __builtin_memcpy(&v, q, sizeof(vec)); // element-aligned only
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VK; ++e)
+                        if (col + e >= col_lo && col + e < col_hi) v[e] = q[e];
+                }
+            }
+            val[j] = v;
+        }
+#pragma unroll
+        for (int j = 0; j < BATCH; ++j) {
+            const int p = tid + (it0 + j) * C::ITEM_THREADS;
+            const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
+            if (it0 + j < ITER && p < TOTP) *reinterpret_cast<vec *>(lds + band * BAND + row * PITCH + col) = val[j];
+        }
+    }
 }
 
 // Inner loops of one stage for one lane: for every K-column chunk kc in [kc_lo, kc_hi) sweep
@@ -203,16 +310,20 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     using vec = typename vec128<T>::type;
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    T *Vs = reinterpret_cast<T *>(smem_raw);
+    // with row-splitting wavefronts `tid` is the lane and the staging below is per wavefront
+    const int group = C::IW > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6) : 0;
+    const int tid = C::IW > 1 ? ((int)threadIdx.x & 63) : (int)threadIdx.x;
+    T *Vs = reinterpret_cast<T *>(smem_raw) + (size_t)group * C::LDS_ELEMS;
     T *Us = Vs + C::NVB * C::VBAND;
-
-    const int tid = threadIdx.x;
     const int W = g.W, H = g.H;
 
-    // ---- decode the work item (block-uniform) ----
-    int item = blockIdx.x;
+    PhaseClock pc;
+    // ---- decode the work item (uniform over the threads that share it) ----
+    int item = (int)blockIdx.x;
+    if (item >= g.total_items) return;
     const int mat = item % (g.nvg * g.nug);
     item /= (g.nvg * g.nug);
+    const int rc = g.rows_per_chunk;
     const int worker = item % g.nworkers_y;
     const int txi = item / g.nworkers_y;
     const int ug = mat % g.nug, vg = mat / g.nug;
@@ -234,7 +345,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         for (; ty < g.nty; ++ty) {
             int lo, hi;
             tile_rows<C>(ty, H, lo, hi);
-            int n = (hi - lo + g.rows_per_chunk - 1) / g.rows_per_chunk;
+            int n = (hi - lo + rc - 1) / rc;
             if (w < n) break;
             w -= n;
         }
@@ -243,10 +354,16 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     }
     int row_lo, row_hi;
     tile_rows<C>(ty, H, row_lo, row_hi);
-    const int clo = row_lo + chunk * g.rows_per_chunk;
-    int chi = clo + g.rows_per_chunk;
+    int clo = row_lo + chunk * rc;
+    int chi = clo + rc;
     if (chi > row_hi) chi = row_hi;
     if (clo >= chi) return; // surplus worker of the rectangle distribution
+    if (C::IW > 1) {
+        // this wavefront's share of the rows, a whole number of staged bands
+        int share = ((chi - clo + C::IW - 1) / C::IW + C::RL - 1) / C::RL * C::RL;
+        clo += group * share;
+        if (clo + share < chi) chi = clo + share;
+    }
 
     const int syb = -(H - 1) + ty * C::TYB;
     const int sxb = -(W - 1) + tx * C::TXB;
@@ -271,7 +388,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
 
     // ---- lane coordinates ----
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = C::IW > 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wx = wave % C::WX, wy = wave / C::WX;
     // x fastest, y slowest: the eight lanes an LDS access serves together then differ in what
     // selects the LEFT address (x, left matrix) and share the right-row address, or differ in
@@ -312,43 +429,35 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             if (h < jj_hi) jj_hi = h;
         }
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
-            __syncthreads(); // everyone is done reading the previous stage
+            if (x0 == xr_lo && yl0 == clo)
+                pc.lap(PH_SETUP);
+            else
+                pc.lap(PH_COMPUTE);
+            item_sync<C>(); // everyone is done reading the previous stage
+            pc.lap(PH_WAIT_SIBLINGS);
             // ---- stage the left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col ----
             {
                 const int xbase = x0 + sxb;
-                constexpr int TOT = C::NVB * (C::RL + 1) * C::PV;
-#pragma unroll
-                for (int idx = tid; idx < TOT; idx += C::NT) {
-                    int col = idx % C::PV;
-                    int t = idx / C::PV;
-                    int row = t % (C::RL + 1);
-                    int band = t / (C::RL + 1);
-                    int v = v_first + band, yl = yl0 + row, xl = xbase + col;
-                    int dst = band * C::VBAND + row * C::PV + col;
-                    T val = T(0);
-                    if (v < g.nV && row < C::RL && yl < chi && (unsigned)xl < (unsigned)W) val = g.V[(size_t)v * HW + (size_t)yl * W + xl];
-                    Vs[dst] = val;
-                }
+                int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
+                int nb = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
+                int c_lo = xbase < 0 ? -xbase : 0;
+                int c_hi = W - xbase < C::PV ? W - xbase : C::PV;
+                stage_bands<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(Vs, g.V + (size_t)v_first * HW, HW, W, nb, 0, rows_ok, yl0, xbase, c_lo,
+                                                                   c_hi, tid);
             }
             // ---- stage the right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col ----
             {
                 const int yr0 = yl0 - syb - C::TYB + 1;
-                constexpr int TOT = C::NUB * (C::RU + 1) * C::PU;
-#pragma unroll
-                for (int idx = tid; idx < TOT; idx += C::NT) {
-                    int col = idx % C::PU;
-                    int t = idx / C::PU;
-                    int row = t % (C::RU + 1);
-                    int band = t / (C::RU + 1);
-                    int u = u_first + band, yr = yr0 + row, xr = x0 + col;
-                    int dst = band * C::UBAND + row * C::PU + col;
-                    T val = T(0);
-                    if (u < u_limit && col < C::KBX && (unsigned)yr < (unsigned)H && xr < W)
-                        val = g.U[(size_t)u * HW + (size_t)yr * W + xr];
-                    Us[dst] = val;
-                }
+                int nb = u_limit - u_first < C::NUB ? u_limit - u_first : C::NUB;
+                int r_lo = yr0 < 0 ? -yr0 : 0;
+                int r_hi = H - yr0 < C::RU + 1 ? H - yr0 : C::RU + 1;
+                int c_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
+                stage_bands<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(Us, g.U + (size_t)u_first * HW, HW, W, nb, r_lo, r_hi, yr0, x0, 0, c_hi,
+                                                                   tid);
             }
-            __syncthreads();
+            pc.lap(PH_STAGING);
+            item_sync<C>();
+            pc.lap(PH_WAIT_STAGED);
 
             // ---- K-column chunks of this stage that overlap this wavefront's x shifts ----
             int kc_lo = 0, kc_hi = C::KBX / K;
@@ -367,11 +476,80 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         }
     }
 
+    pc.lap(PH_COMPUTE);
     // ---- write the register tiles ----
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     const size_t out_area = (size_t)Sx * Sy;
     const int ox0 = sxw + lx * B + (W - 1);
     const int oy0 = syw + ly * A + (H - 1);
+    if constexpr (C::IW > 1) {
+        // Add the partial tiles of the IW wavefronts. In pass q wavefront w ends up with the
+        // sums of tile row q*IW + w: everyone deposits rows q*IW .. q*IW+IW-1, then reads back
+        // all IW versions of its own row (in wavefront order, so the result is deterministic).
+        T *red = reinterpret_cast<T *>(smem_raw);
+        constexpr int RR = C::RED_ROW;
+#pragma unroll
+        for (int q = 0; q < A / C::IW; ++q) {
+            __syncthreads(); // bands, or the previous pass, are no longer read
+#pragma unroll
+            for (int o = 0; o < C::IW; ++o) {
+                T *dst = red + ((size_t)(o * C::IW + group) * 64 + lane) * RR;
+#pragma unroll
+                for (int i = 0; i < NV; ++i)
+#pragma unroll
+                    for (int n = 0; n < NU; ++n)
+#pragma unroll
+                        for (int b = 0; b < B; b += VK) {
+                            vec piece;
+#pragma unroll
+                            for (int e = 0; e < VK; ++e) piece[e] = acc[i][n][q * C::IW + o][b + e];
+                            *reinterpret_cast<vec *>(dst + (i * NU + n) * B + b) = piece;
+                        }
+            }
+            __syncthreads();
+            T sum[NV][NU][B];
+#pragma unroll
+            for (int src = 0; src < C::IW; ++src) {
+                const T *from = red + ((size_t)(group * C::IW + src) * 64 + lane) * RR;
+#pragma unroll
+                for (int i = 0; i < NV; ++i)
+#pragma unroll
+                    for (int n = 0; n < NU; ++n)
+#pragma unroll
+                        for (int b = 0; b < B; b += VK) {
+                            vec piece = *reinterpret_cast<const vec *>(from + (i * NU + n) * B + b);
+#pragma unroll
+                            for (int e = 0; e < VK; ++e) sum[i][n][b + e] = src == 0 ? piece[e] : sum[i][n][b + e] + piece[e];
+                        }
+            }
+            const int oy = oy0 + q * C::IW + group;
+            if (oy < 0 || oy >= Sy) continue;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = v_first + lv * NV + i;
+                if (v >= g.nV) continue;
+#pragma unroll
+                for (int n = 0; n < NU; ++n) {
+                    const int u = u_first + lu * NU + n;
+                    if (u >= u_limit) continue;
+                    const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
+                    T *o = g.out + mat_index * out_area + (size_t)oy * Sx;
+#pragma unroll
+                    for (int b = 0; b < B; ++b) {
+                        const int ox = ox0 + b;
+                        if (ox < 0 || ox >= Sx) continue;
+                        if (g.atomic)
+                            atomic_add(o + ox, sum[i][n][b]);
+                        else
+                            o[ox] = sum[i][n][b];
+                    }
+                }
+            }
+        }
+        pc.lap(PH_OUTPUT);
+        pc.flush();
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = v_first + lv * NV + i;
@@ -399,6 +577,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             }
         }
     }
+    pc.lap(PH_OUTPUT);
+    pc.flush();
 }
 
 // fills n elements with zero (a plain kernel rather than a memset node, so callers may capture it)

@@ -16,6 +16,12 @@ using G_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 2, 2, 18, 8, 2>;
 using G_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 2, 2, 9, 4, 2>;
 using G_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 2, 2, 9, 8, 2>;
 using G_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 2, 2, 18, 8, 2>;
+// four independent wavefronts per workgroup (last parameter)
+using I_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 18, 4, 2, 4>;
+using I_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 10, 8, 4, 4>;
+using I_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 9, 4, 2, 4>;
+using I_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 1, 1, 9, 4, 2, 4>;
+using I_48_v8u8 = EngineCfg<double, 4, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 10, 4, 4, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
@@ -27,6 +33,11 @@ static const EngineSpec specs[] = {
     make_spec<G_88_u16>("f64_a8b8_lr16"),
     make_spec<G_88_v8u8>("f64_a8b8_ll8lr8"),
     make_spec<G_88_v4u4>("f64_a8b8_ll4lr4"),
+    make_spec<I_88>("f64_a8b8_i4"),
+    make_spec<I_44>("f64_a4b4_i4"),
+    make_spec<I_88_v8u8>("f64_a8b8_ll8lr8_i4"),
+    make_spec<I_88_v4u4>("f64_a8b8_ll4lr4_i4"),
+    make_spec<I_48_v8u8>("f64_a4b8_ll8lr8_i4"),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {
@@ -35,3 +46,8 @@ const EngineSpec *engine_specs_f64(int *count) {
 }
 
 } // namespace xcorr
+
+#ifdef XCORR_ENGINE_PROFILE
+// profile builds only: copies out and clears the per-phase cycle table of the f64 kernels
+extern "C" int xcorr_debug_engine_profile_f64(unsigned long long *out) { return (int)xcorr::engine_profile_read(out); }
+#endif

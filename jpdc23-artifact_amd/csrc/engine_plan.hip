@@ -3,6 +3,8 @@
 // into work items, clears the output when it splits on its own, launches and
 // records the geometry.
 #include <cmath>
+#include <cstdlib>
+#include <cstring>
 
 #include "engine_registry.hpp"
 
@@ -48,7 +50,7 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double cost = waste_x * waste_y / (util_v * util_u) * issue;
     if (s.LV * s.LU > 1) cost *= 2.0;
     if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
-    if (s.WX * s.WY < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
+    if (s.WX * s.WY * s.IW < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
     if (rq.y_shifts > 1) cost *= 1.0 + 3.0 * log2_ratio(s.A, rq.y_shifts);
     if (rq.left_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NV, rq.left_mats);
     if (rq.right_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NU, rq.right_mats);
@@ -110,7 +112,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
             const long target = 32L * device_cus();
             long chunks_wanted = (target + tiles - 1) / tiles;
             // a work item should span at least two staged bands of left rows
-            long most = rq.H / (2 * best->RL);
+            long most = rq.H / (2 * best->RL * best->IW);
             if (chunks_wanted > most) chunks_wanted = most;
             if (chunks_wanted > 1) {
                 rc = ceil_div(rq.H, (int)chunks_wanted);
@@ -150,9 +152,10 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         plan.nworkers_y = plan.nty * max_chunks;
     else
         plan.nworkers_y = (int)total_chunks;
-    long grid = (long)plan.nvg * plan.nug * plan.nworkers_y * plan.ntx;
-    if (grid <= 0 || grid > 0x7fffffffL) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: grid of %ld blocks is out of range", rq.family, grid);
-    plan.grid = (unsigned)grid;
+    long items = (long)plan.nvg * plan.nug * plan.nworkers_y * plan.ntx;
+    if (items <= 0 || items > 0x7fffffffL) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: %ld work items are out of range", rq.family, items);
+    plan.total_items = (int)items;
+    plan.grid = (unsigned)items;
     return XCORR_OK;
 }
 
@@ -175,6 +178,7 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     a.nworkers_y = plan.nworkers_y;
     a.nvg = plan.nvg;
     a.nug = plan.nug;
+    a.total_items = plan.total_items;
     if (plan.zero_fill) {
         size_t n = (size_t)(2 * rq.W - 1) * (2 * rq.H - 1) * (rq.group_m > 0 ? (size_t)rq.nU : (size_t)rq.nV * rq.nU);
         size_t blocks = (n + 256 * 8 - 1) / (256 * 8);

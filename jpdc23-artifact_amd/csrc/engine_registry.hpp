@@ -18,6 +18,7 @@ struct EngineSpec {
     int A, B, K, NV, NU;
     int LX, LY, LV, LU;
     int WX, WY, RL, KBX;
+    int IW; // independent wavefronts (work items) per workgroup
     int lds_bytes;
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
@@ -53,7 +54,8 @@ constexpr EngineSpec make_spec(const char *name) {
                       C::LY,  C::LV,
                       C::LU,  C::WX,
                       C::WY,  C::RL,
-                      C::KBX, C::LDS_BYTES,
+                      C::KBX, C::IW,
+                      C::LDS_BYTES,
                       C::NT,  &launch_engine<C>};
 }
 
@@ -81,7 +83,7 @@ struct EngineRequest {
 struct EnginePlan {
     const EngineSpec *spec;
     int ntx, nty, nworkers_y, nvg, nug;
-    int rows_per_chunk, dist, atomic;
+    int rows_per_chunk, dist, atomic, total_items;
     bool zero_fill;
     unsigned grid;
 };
