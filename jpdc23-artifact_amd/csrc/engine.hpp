@@ -49,24 +49,26 @@ struct EngineArgs {
     int total_items;    // nvg * nug * nworkers_y * ntx
 };
 
-// IW_ > 1: the IW_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
-// matrices and split its left rows among themselves: each stages its own LDS bands, runs without
-// workgroup barriers, and the partial sums are added through LDS before the tile is written. This
-// divides the longest work item of a launch by IW_ without atomics, which is what small matrices
-// laid over lanes need: their central tiles would otherwise run long after the rest has finished.
+// WZ_ > 1: the WZ_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
+// matrices and split its left rows: a stage holds WZ_ (or a multiple) groups of G left rows, staged
+// by all threads together, and each wavefront sweeps its own groups. The wavefronts do the same
+// amount of work per stage, so the barriers around a stage cost little (wavefronts that own
+// different shift tiles skip different parts of a stage and wait for each other), the block tile
+// is as small as the wavefront tile (less work on partial overlaps), and the longest work item
+// of a launch is WZ_ times shorter. The partial sums are added through LDS before the tile is
+// written, or added atomically by each wavefront when the output is accumulated atomically anyway.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
-          int RL_, int KBX_, int MINB_, int IW_ = 1>
+          int RL_, int KBX_, int MINB_, int WZ_ = 1>
 struct EngineCfg {
     using value_type = T;
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
-    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, IW = IW_;
+    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_;
     static constexpr int VK = 16 / (int)sizeof(T); // elements per 128-bit LDS access
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
-    static constexpr int NWAVES = WX * WY, NT = 64 * NWAVES * IW;
-    static constexpr int ITEM_THREADS = 64 * NWAVES; // threads that cooperate on one work item
-    static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
+    static constexpr int NWAVES = WX * WY * WZ, NT = 64 * NWAVES;
+        static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
     static constexpr int VWIN = B + K - 1;
     static constexpr int VWIN_VECS = (VWIN + VK - 1) / VK;
     static constexpr int KVECS = K / VK;
@@ -84,10 +86,11 @@ struct EngineCfg {
     static constexpr int LDS_ELEMS = NVB * VBAND + NUB * UBAND;
     // in-block reduction: one output row of the tile per wavefront and pass, [owner][source][lane][RED_ROW]
     static constexpr int RED_ROW = NV * NU * B;
-    static constexpr int RED_ELEMS = IW > 1 ? IW * IW * 64 * RED_ROW : 0;
-    static constexpr int LDS_BYTES = (LDS_ELEMS * IW > RED_ELEMS ? LDS_ELEMS * IW : RED_ELEMS) * (int)sizeof(T);
+    static constexpr int RED_ELEMS = WZ > 1 ? WZ * WZ * 64 * RED_ROW : 0;
+    static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
-    static_assert(IW == 1 || (WX == 1 && WY == 1 && A % IW == 0), "row-splitting wavefronts share one wavefront tile");
+    static_assert(WZ == 1 || (WX == 1 && WY == 1 && A % WZ == 0), "row-splitting wavefronts share one wavefront tile");
+    static_assert((RL / (A_ + 1)) % WZ == 0, "every wavefront gets the same number of row groups per stage");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
@@ -106,14 +109,15 @@ struct vec128<double> {
 // Cycle accounting per phase of engine_kernel, compiled in with -DXCORR_ENGINE_PROFILE only (a
 // tuning aid: every wavefront adds the shader-clock cycles it spent per phase to a device-side
 // table that engine_profile_read() copies out and clears).
-enum EnginePhase { PH_SETUP, PH_WAIT_SIBLINGS, PH_STAGING, PH_WAIT_STAGED, PH_COMPUTE, PH_OUTPUT, PH_COUNT };
+enum EnginePhase { PH_SETUP, PH_WAIT_SIBLINGS, PH_STAGING, PH_WAIT_STAGED, PH_COMPUTE, PH_OUTPUT, PH_DECODE, PH_COUNT };
 #ifdef XCORR_ENGINE_PROFILE
-static __device__ unsigned long long engine_profile[PH_COUNT + 2]; // phases, wavefronts, first-to-last cycles
+static __device__ unsigned long long engine_profile[PH_COUNT + 3]; // phases, wavefronts, first-to-last cycles, same in 100 MHz ticks
 struct PhaseClock {
-    long long t0, t, acc[PH_COUNT];
+    long long t0, t, w0, acc[PH_COUNT];
     __device__ __forceinline__ PhaseClock() {
         for (int i = 0; i < PH_COUNT; ++i) acc[i] = 0;
         t0 = t = (long long)clock64();
+        w0 = (long long)wall_clock64();
     }
     __device__ __forceinline__ void lap(int phase) {
         long long now = (long long)clock64();
@@ -125,13 +129,14 @@ struct PhaseClock {
             for (int i = 0; i < PH_COUNT; ++i) atomicAdd(&engine_profile[i], (unsigned long long)acc[i]);
             atomicAdd(&engine_profile[PH_COUNT], 1ull);
             atomicAdd(&engine_profile[PH_COUNT + 1], (unsigned long long)(t - t0));
+            atomicAdd(&engine_profile[PH_COUNT + 2], (unsigned long long)((long long)wall_clock64() - w0));
         }
     }
 };
 static inline hipError_t engine_profile_read(unsigned long long *out) {
     hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(engine_profile), sizeof(engine_profile));
     if (e != hipSuccess) return e;
-    unsigned long long zero[PH_COUNT + 2] = {};
+    unsigned long long zero[PH_COUNT + 3] = {};
     return hipMemcpyToSymbol(HIP_SYMBOL(engine_profile), zero, sizeof(zero));
 }
 #else
@@ -153,18 +158,6 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
     hi = h < H ? h : H;
 }
 
-// Orders the LDS writes of a stage before its reads (and the reads before the next stage's
-// writes) among the threads that share a work item: a workgroup barrier, or nothing but a
-// compiler fence when the item belongs to a single wavefront (the LDS serves the accesses of
-// one wavefront in program order).
-template <class C>
-__device__ __forceinline__ void item_sync() {
-    if (C::IW > 1)
-        __builtin_amdgcn_wave_barrier();
-    else
-        __syncthreads();
-}
-
 // Fills the LDS image of NB bands (ROWS rows of PITCH elements, BAND elements apart) from NB
 // matrices that are `mat_stride` elements apart in global memory. Image element (band, row, col)
 // is src[band][row0 + row][col0 + col] if band < nbands, row_lo <= row < row_hi and
@@ -177,7 +170,7 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     constexpr int VK = C::VK, PP = PITCH / VK, TOTP = NB * ROWS * PP;
-    constexpr int ITER = (TOTP + C::ITEM_THREADS - 1) / C::ITEM_THREADS;
+    constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
     constexpr int BATCH = ITER < 8 ? ITER : 8;
     static_assert(PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
 #pragma unroll
@@ -185,7 +178,7 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
         vec val[BATCH];
 #pragma unroll
         for (int j = 0; j < BATCH; ++j) {
-            const int p = tid + (it0 + j) * C::ITEM_THREADS;
+            const int p = tid + (it0 + j) * C::NT;
             const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
             vec v;
 #pragma unroll
@@ -204,7 +197,7 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
         }
 #pragma unroll
         for (int j = 0; j < BATCH; ++j) {
-            const int p = tid + (it0 + j) * C::ITEM_THREADS;
+            const int p = tid + (it0 + j) * C::NT;
             const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
             if (it0 + j < ITER && p < TOTP) *reinterpret_cast<vec *>(lds + band * BAND + row * PITCH + col) = val[j];
         }
@@ -310,10 +303,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     using vec = typename vec128<T>::type;
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-    // with row-splitting wavefronts `tid` is the lane and the staging below is per wavefront
-    const int group = C::IW > 1 ? __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6) : 0;
-    const int tid = C::IW > 1 ? ((int)threadIdx.x & 63) : (int)threadIdx.x;
-    T *Vs = reinterpret_cast<T *>(smem_raw) + (size_t)group * C::LDS_ELEMS;
+    const int tid = (int)threadIdx.x;
+    const int group = C::WZ > 1 ? __builtin_amdgcn_readfirstlane(tid >> 6) : 0; // which share of the rows
+    T *Vs = reinterpret_cast<T *>(smem_raw);
     T *Us = Vs + C::NVB * C::VBAND;
     const int W = g.W, H = g.H;
 
@@ -327,44 +319,40 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const int worker = item % g.nworkers_y;
     const int txi = item / g.nworkers_y;
     const int ug = mat % g.nug, vg = mat / g.nug;
-    // x tiles are visited centre-out: the block index order is the dispatch order and
-    // central tiles have the longest overlaps
-    const int txc = g.ntx / 2;
+    // x and y tiles are visited centre-out: the block index order is the dispatch order, and
+    // central tiles have the longest overlaps, so the longest work items start first
+    const int txc = g.ntx / 2, tyc = g.nty / 2;
     const int tx = (txi & 1) ? txc - (txi + 1) / 2 : txc + txi / 2;
 
-    int ty, chunk;
+    int tyi, chunk;
     if (g.dist == 0) {
-        ty = worker;
+        tyi = worker;
         chunk = 0;
     } else if (g.dist == 1) {
-        ty = worker % g.nty;
+        tyi = worker % g.nty;
         chunk = worker / g.nty;
     } else {
         int w = worker;
-        ty = 0;
-        for (; ty < g.nty; ++ty) {
+        tyi = 0;
+        for (; tyi < g.nty; ++tyi) {
             int lo, hi;
-            tile_rows<C>(ty, H, lo, hi);
+            tile_rows<C>((tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2, H, lo, hi);
             int n = (hi - lo + rc - 1) / rc;
             if (w < n) break;
             w -= n;
         }
         chunk = w;
-        if (ty >= g.nty) return;
+        if (tyi >= g.nty) return;
     }
+    const int ty = (tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2;
     int row_lo, row_hi;
     tile_rows<C>(ty, H, row_lo, row_hi);
-    int clo = row_lo + chunk * rc;
+    const int clo = row_lo + chunk * rc;
     int chi = clo + rc;
     if (chi > row_hi) chi = row_hi;
     if (clo >= chi) return; // surplus worker of the rectangle distribution
-    if (C::IW > 1) {
-        // this wavefront's share of the rows, a whole number of staged bands
-        int share = ((chi - clo + C::IW - 1) / C::IW + C::RL - 1) / C::RL * C::RL;
-        clo += group * share;
-        if (clo + share < chi) chi = clo + share;
-    }
 
+    pc.lap(PH_DECODE);
     const int syb = -(H - 1) + ty * C::TYB;
     const int sxb = -(W - 1) + tx * C::TXB;
 
@@ -388,7 +376,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
 
     // ---- lane coordinates ----
     const int lane = tid & 63;
-    const int wave = C::IW > 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = C::WZ > 1 ? 0 : __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wx = wave % C::WX, wy = wave / C::WX;
     // x fastest, y slowest: the eight lanes an LDS access serves together then differ in what
     // selects the LEFT address (x, left matrix) and share the right-row address, or differ in
@@ -427,13 +415,19 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             if (first > 0) jj_lo = first / C::G;
             int h = last < 0 ? 0 : last / C::G + 1;
             if (h < jj_hi) jj_hi = h;
+            if (C::WZ > 1) {
+                // this wavefront's groups of the stage
+                constexpr int M = C::RL / C::G / C::WZ;
+                if (jj_lo < group * M) jj_lo = group * M;
+                if (jj_hi > (group + 1) * M) jj_hi = (group + 1) * M;
+            }
         }
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
             if (x0 == xr_lo && yl0 == clo)
                 pc.lap(PH_SETUP);
             else
                 pc.lap(PH_COMPUTE);
-            item_sync<C>(); // everyone is done reading the previous stage
+            __syncthreads(); // everyone is done reading the previous stage
             pc.lap(PH_WAIT_SIBLINGS);
             // ---- stage the left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col ----
             {
@@ -456,7 +450,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                                                                    tid);
             }
             pc.lap(PH_STAGING);
-            item_sync<C>();
+            __syncthreads();
             pc.lap(PH_WAIT_STAGED);
 
             // ---- K-column chunks of this stage that overlap this wavefront's x shifts ----
@@ -482,18 +476,18 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const size_t out_area = (size_t)Sx * Sy;
     const int ox0 = sxw + lx * B + (W - 1);
     const int oy0 = syw + ly * A + (H - 1);
-    if constexpr (C::IW > 1) {
-        // Add the partial tiles of the IW wavefronts. In pass q wavefront w ends up with the
-        // sums of tile row q*IW + w: everyone deposits rows q*IW .. q*IW+IW-1, then reads back
-        // all IW versions of its own row (in wavefront order, so the result is deterministic).
+    if (C::WZ > 1 && !g.atomic) {
+        // Add the partial tiles of the WZ wavefronts. In pass q wavefront w ends up with the
+        // sums of tile row q*WZ + w: everyone deposits rows q*WZ .. q*WZ+WZ-1, then reads back
+        // all WZ versions of its own row (in wavefront order, so the result is deterministic).
         T *red = reinterpret_cast<T *>(smem_raw);
         constexpr int RR = C::RED_ROW;
 #pragma unroll
-        for (int q = 0; q < A / C::IW; ++q) {
+        for (int q = 0; q < A / C::WZ; ++q) {
             __syncthreads(); // bands, or the previous pass, are no longer read
 #pragma unroll
-            for (int o = 0; o < C::IW; ++o) {
-                T *dst = red + ((size_t)(o * C::IW + group) * 64 + lane) * RR;
+            for (int o = 0; o < C::WZ; ++o) {
+                T *dst = red + ((size_t)(o * C::WZ + group) * 64 + lane) * RR;
 #pragma unroll
                 for (int i = 0; i < NV; ++i)
 #pragma unroll
@@ -502,15 +496,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                         for (int b = 0; b < B; b += VK) {
                             vec piece;
 #pragma unroll
-                            for (int e = 0; e < VK; ++e) piece[e] = acc[i][n][q * C::IW + o][b + e];
+                            for (int e = 0; e < VK; ++e) piece[e] = acc[i][n][q * C::WZ + o][b + e];
                             *reinterpret_cast<vec *>(dst + (i * NU + n) * B + b) = piece;
                         }
             }
             __syncthreads();
             T sum[NV][NU][B];
 #pragma unroll
-            for (int src = 0; src < C::IW; ++src) {
-                const T *from = red + ((size_t)(group * C::IW + src) * 64 + lane) * RR;
+            for (int src = 0; src < C::WZ; ++src) {
+                const T *from = red + ((size_t)(group * C::WZ + src) * 64 + lane) * RR;
 #pragma unroll
                 for (int i = 0; i < NV; ++i)
 #pragma unroll
@@ -522,7 +516,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                             for (int e = 0; e < VK; ++e) sum[i][n][b + e] = src == 0 ? piece[e] : sum[i][n][b + e] + piece[e];
                         }
             }
-            const int oy = oy0 + q * C::IW + group;
+            const int oy = oy0 + q * C::WZ + group;
             if (oy < 0 || oy >= Sy) continue;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
@@ -550,6 +544,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         pc.flush();
         return;
     }
+    // (row-splitting wavefronts of an atomically accumulated tile add their partial sums directly)
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = v_first + lv * NV + i;

@@ -5,58 +5,51 @@
 // plain v_fmac_f32 only reaches the vector peak with at least two wavefronts issuing per
 // SIMD, and an even number of resident wavefronts measured best) and its LDS bands at or
 // below ~40 KB per four-wavefront block so four blocks share a CU.
+// Names: a<y shifts>b<x shifts> per lane, r/l = right/left matrices per lane, lr/ll = lanes
+// laid over right/left matrices.
 #include "engine_registry.hpp"
 
 namespace xcorr {
 
-//                          T      A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB
-// one output row per lane (families: shuffle, split-row, multimat-right, multimat-both)
+//                             T      A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB WZ
+// one output row per lane (families: shuffle, split-row, multimat-right, multimat-both); four
+// wavefronts tile 2x2 over the shifts
 using R_1x1 = EngineCfg<float, 1, 8, 4, 1, 1, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_1x4 = EngineCfg<float, 1, 8, 4, 1, 4, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_2x2 = EngineCfg<float, 1, 8, 4, 2, 2, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
-// grouped (several y shifts per lane)
-using G_88 = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 2, 2, 18, 32, 4>;
-using G_88_w1 = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 18, 32, 4>;
-using G_44 = EngineCfg<float, 4, 4, 4, 1, 1, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
-using G_44_w1 = EngineCfg<float, 4, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 20, 32, 4>;
-using G_88_u4 = EngineCfg<float, 8, 8, 4, 1, 1, 4, 4, 1, 4, 2, 2, 18, 16, 4>;
-using G_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 2, 2, 9, 8, 4>;
-using G_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 2, 2, 9, 16, 4>;
-using G_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 2, 2, 18, 16, 4>;
+// several matrices per lane (the reference's left/right_matrices_per_thread), 2x2 wavefronts
 using G_48_n2 = EngineCfg<float, 4, 8, 4, 1, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
 using G_44_n22 = EngineCfg<float, 4, 4, 4, 2, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
-// four independent wavefronts per workgroup (last parameter), one tile and one set of bands each
-using I_88 = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 18, 8, 4, 4>;
-using I_88b = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 9, 16, 4, 4>;
-using I_44 = EngineCfg<float, 4, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 20, 16, 4, 4>;
-using I_88_u4 = EngineCfg<float, 8, 8, 4, 1, 1, 4, 4, 1, 4, 1, 1, 9, 8, 4, 4>;
-using I_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 9, 8, 4, 4>;
-using I_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 9, 8, 4, 4>;
-using I_48 = EngineCfg<float, 4, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 20, 16, 4, 4>;
-using I_84 = EngineCfg<float, 8, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 18, 16, 4, 4>;
+// grouped tiles: four wavefronts share one tile and its bands and take one group of rows each per
+// stage (WZ = 4). Lanes over shifts only ...
+using Z_84 = EngineCfg<float, 8, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
+using Z_88 = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
+using Z_44 = EngineCfg<float, 4, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 20, 32, 4, 4>;
+// ... and lanes over right matrices (one_to_many, n_to_mn) or over pairs (n_to_m) of small matrices
+using Z_84_u4 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 4, 1, 4, 1, 1, 36, 16, 4, 4>;
+using Z_88_u4 = EngineCfg<float, 8, 8, 4, 1, 1, 4, 4, 1, 4, 1, 1, 36, 16, 4, 4>;
+using Z_84_u16 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 4, 4>;
+using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 4, 4>;
+using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
+using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
+using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 36, 8, 4, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),
     make_spec<R_1x4>("f32_a1b8_r4"),
     make_spec<R_2x2>("f32_a1b8_l2r2"),
-    make_spec<G_88>("f32_a8b8"),
-    make_spec<G_88_w1>("f32_a8b8_w1"),
-    make_spec<G_44>("f32_a4b4"),
-    make_spec<G_44_w1>("f32_a4b4_w1"),
-    make_spec<G_88_u4>("f32_a8b8_lr4"),
-    make_spec<G_88_u16>("f32_a8b8_lr16"),
-    make_spec<G_88_v8u8>("f32_a8b8_ll8lr8"),
-    make_spec<G_88_v4u4>("f32_a8b8_ll4lr4"),
     make_spec<G_48_n2>("f32_a4b8_r2"),
     make_spec<G_44_n22>("f32_a4b4_l2r2"),
-    make_spec<I_88>("f32_a8b8_i4"),
-    make_spec<I_88b>("f32_a8b8_i4_rl9"),
-    make_spec<I_44>("f32_a4b4_i4"),
-    make_spec<I_88_u4>("f32_a8b8_lr4_i4"),
-    make_spec<I_88_v8u8>("f32_a8b8_ll8lr8_i4"),
-    make_spec<I_88_v4u4>("f32_a8b8_ll4lr4_i4"),
-    make_spec<I_48>("f32_a4b8_i4"),
-    make_spec<I_84>("f32_a8b4_i4"),
+    make_spec<Z_84>("f32_a8b4"),
+    make_spec<Z_88>("f32_a8b8"),
+    make_spec<Z_44>("f32_a4b4"),
+    make_spec<Z_84_u4>("f32_a8b4_lr4"),
+    make_spec<Z_88_u4>("f32_a8b8_lr4"),
+    make_spec<Z_84_u16>("f32_a8b4_lr16"),
+    make_spec<Z_88_u16>("f32_a8b8_lr16"),
+    make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4"),
+    make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4"),
+    make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8"),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {

@@ -6,38 +6,33 @@
 
 namespace xcorr {
 
-//                           T       A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB
+//                              T       A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB WZ
+// one output row per lane, 2x2 wavefronts over the shifts
 using R_1x1 = EngineCfg<double, 1, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
 using R_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
-using G_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 18, 16, 2>;
-using G_88_w1 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 18, 16, 2>;
-using G_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 2, 2, 20, 16, 4>;
-using G_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 2, 2, 18, 8, 2>;
-using G_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 2, 2, 9, 4, 2>;
-using G_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 2, 2, 9, 8, 2>;
-using G_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 2, 2, 18, 8, 2>;
-// four independent wavefronts per workgroup (last parameter)
-using I_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 18, 4, 2, 4>;
-using I_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 10, 8, 4, 4>;
-using I_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 9, 4, 2, 4>;
-using I_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 1, 1, 9, 4, 2, 4>;
-using I_48_v8u8 = EngineCfg<double, 4, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 10, 4, 4, 4>;
+// grouped tiles: four wavefronts share one tile and its bands and take one group of rows each per stage
+using Z_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 2, 4>;
+using Z_84 = EngineCfg<double, 8, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 4, 4>;
+using Z_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 20, 16, 4, 4>;
+using Z_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 1, 1, 36, 8, 2, 4>;
+using Z_84_u4 = EngineCfg<double, 8, 4, 2, 1, 1, 4, 4, 1, 4, 1, 1, 36, 8, 4, 4>;
+using Z_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 2, 4>;
+using Z_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 2, 4>;
+using Z_84_v4u4 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
+using Z_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 36, 8, 2, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
     make_spec<R_2x2>("f64_a1b4_l2r2"),
-    make_spec<G_88>("f64_a8b8"),
-    make_spec<G_88_w1>("f64_a8b8_w1"),
-    make_spec<G_44>("f64_a4b4"),
-    make_spec<G_88_u4>("f64_a8b8_lr4"),
-    make_spec<G_88_u16>("f64_a8b8_lr16"),
-    make_spec<G_88_v8u8>("f64_a8b8_ll8lr8"),
-    make_spec<G_88_v4u4>("f64_a8b8_ll4lr4"),
-    make_spec<I_88>("f64_a8b8_i4"),
-    make_spec<I_44>("f64_a4b4_i4"),
-    make_spec<I_88_v8u8>("f64_a8b8_ll8lr8_i4"),
-    make_spec<I_88_v4u4>("f64_a8b8_ll4lr4_i4"),
-    make_spec<I_48_v8u8>("f64_a4b8_ll8lr8_i4"),
+    make_spec<Z_88>("f64_a8b8"),
+    make_spec<Z_84>("f64_a8b4"),
+    make_spec<Z_44>("f64_a4b4"),
+    make_spec<Z_88_u4>("f64_a8b8_lr4"),
+    make_spec<Z_84_u4>("f64_a8b4_lr4"),
+    make_spec<Z_88_u16>("f64_a8b8_lr16"),
+    make_spec<Z_88_v4u4>("f64_a8b8_ll4lr4"),
+    make_spec<Z_84_v4u4>("f64_a8b4_ll4lr4"),
+    make_spec<Z_88_v8u8>("f64_a8b8_ll8lr8"),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {

@@ -27,35 +27,61 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)); }
 
-// Relative cost of running the request on a specialisation, calibrated on MI355X sweeps:
-//   * work issued for partial overlaps at tile edges. Wavefronts skip what cannot overlap
-//     their own tile, but the waves of a block meet at a barrier after every staged band,
-//     so both the wavefront tile and the block tile count;
+// Relative cost of running the request on a specialisation, calibrated on MI355X sweeps of
+// 64x64 ... 1024x1024 matrices in all four modes:
+//   * work issued for partial overlaps at tile edges: a wavefront skips what cannot overlap its
+//     own tile, but wavefronts that own different shift tiles of one block wait for each other
+//     after every staged band, so for those both the wavefront tile and the block tile count;
 //   * lanes idling over matrices that do not exist;
-//   * issue slots lost to LDS reads: a read plus the wait that guards it displace about nine
-//     fp32 FMA slots (half as many fp64 ones) of the wavefront that issues them;
-//   * lanes laid over matrices stage many small bands and write one matrix per lane.
+//   * the issue rate of the tile: one-row tiles lose issue slots to LDS reads (a read plus the
+//     wait that guards it displace about nine fp32 FMA slots, half as many fp64 ones); among
+//     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower;
+//   * lanes laid over more than four matrices stage many small bands: +12.5 % per doubling.
 // Hints scale the cost so the nearest specialisation wins without excluding the others.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
-    // geometric mean of the wavefront-tile and block-tile overheads
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
     double waste_y = std::sqrt((double)(rq.H + s.TYW()) * (rq.H + s.TYB())) / rq.H;
     int nu = rq.group_m > 0 ? rq.group_m : rq.nU;
     double util_v = (double)rq.nV / ((double)ceil_div(rq.nV, s.NVB()) * s.NVB());
     double util_u = (double)nu / ((double)ceil_div(nu, s.NUB()) * s.NUB());
-    int vk = 16 / s.elem_bytes;
-    double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
-    double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
-    double issue = 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
-    double cost = waste_x * waste_y / (util_v * util_u) * issue;
-    if (s.LV * s.LU > 1) cost *= 2.0;
+    double cost = waste_x * waste_y / (util_v * util_u);
+    if (s.A == 1) {
+        int vk = 16 / s.elem_bytes;
+        double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
+        double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
+        cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
+    } else if (s.A == 8 && s.B == 8) {
+        cost *= s.elem_bytes == 4 ? 1.08 : 1.0;
+    } else if (s.A == 4 && s.B == 4) {
+        cost *= 1.08;
+    }
+    double matrix_lanes = std::log2((double)(s.LV * s.LU));
+    if (matrix_lanes > 2) cost *= 1.0 + 0.125 * (matrix_lanes - 2);
     if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
-    if (s.WX * s.WY * s.IW < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
+    if (s.WX * s.WY * s.WZ < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
+    if (s.A > 1 && s.WZ == 1) cost *= 1.1; // shift-tiled blocks wait at the barriers of partial stages
     if (rq.y_shifts > 1) cost *= 1.0 + 3.0 * log2_ratio(s.A, rq.y_shifts);
     if (rq.left_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NV, rq.left_mats);
     if (rq.right_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NU, rq.right_mats);
-    if (rq.waves) cost *= 1.0 + 0.05 * log2_ratio(s.WX * s.WY, rq.waves);
+    if (rq.waves) cost *= 1.0 + 0.05 * log2_ratio(s.WX * s.WY * s.WZ, rq.waves);
     return cost;
+}
+
+// Number of (y tile, chunk) workers when every y tile's rows are cut into chunks of rc rows.
+static long count_chunks(const EngineSpec &s, int H, int nty, int rc, int *max_chunks) {
+    long total = 0;
+    int most = 0;
+    for (int ty = 0; ty < nty; ++ty) {
+        int syb = -(H - 1) + ty * s.TYB();
+        int lo = syb > 0 ? syb : 0;
+        int hi = syb + s.TYB() - 1 + H;
+        if (hi > H) hi = H;
+        int n = ceil_div(hi - lo, rc);
+        if (n > most) most = n;
+        total += n;
+    }
+    if (max_chunks) *max_chunks = most;
+    return total;
 }
 
 int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
@@ -105,19 +131,20 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         plan.atomic = 1;
         plan.zero_fill = false;
     } else {
-        // lanes laid over matrices write one result matrix per lane: their atomics would not
-        // coalesce, so such tiles are never split by the planner itself
+        // Few tiles: cut the reduction into chunks of whole staged bands (at least two per item)
+        // until the launch has about 64 work items per CU; finer items even out the last wave of
+        // blocks, coarser ones save atomics (measured on 1024x1024: 16 per CU is 10 % slower).
+        // Lanes laid over matrices write one result matrix per lane: their atomics would not
+        // coalesce, so such tiles are never split by the planner itself.
         const bool split_ok = rq.may_split && best->LV * best->LU == 1;
-        if (rc <= 0 && split_ok) {
-            const long target = 32L * device_cus();
-            long chunks_wanted = (target + tiles - 1) / tiles;
-            // a work item should span at least two staged bands of left rows
-            long most = rq.H / (2 * best->RL * best->IW);
-            if (chunks_wanted > most) chunks_wanted = most;
-            if (chunks_wanted > 1) {
-                rc = ceil_div(rq.H, (int)chunks_wanted);
-                rc = ceil_div(rc, best->RL) * best->RL;
+        if (rc <= 0 && split_ok && tiles < 24L * device_cus()) {
+            const long target = 64L * device_cus();
+            const long per_tile_column = (long)plan.ntx * plan.nvg * plan.nug;
+            for (int k = rq.H / best->RL; k >= 2; --k) {
+                rc = k * best->RL;
+                if (per_tile_column * count_chunks(*best, rq.H, plan.nty, rc, nullptr) >= target) break;
             }
+            if (rc <= 0) rc = rq.H;
         }
         if (rc <= 0 || rc >= rq.H || !rq.may_split) {
             rc = rq.H;
@@ -136,16 +163,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
 
     // workers along y: (y tile, chunk) pairs
     int max_chunks = 0;
-    long total_chunks = 0;
-    for (int ty = 0; ty < plan.nty; ++ty) {
-        int syb = -(rq.H - 1) + ty * best->TYB();
-        int lo = syb > 0 ? syb : 0;
-        int hi = syb + best->TYB() - 1 + rq.H;
-        if (hi > rq.H) hi = rq.H;
-        int n = ceil_div(hi - lo, rc);
-        if (n > max_chunks) max_chunks = n;
-        total_chunks += n;
-    }
+    long total_chunks = count_chunks(*best, rq.H, plan.nty, rc, &max_chunks);
     if (dist == 0)
         plan.nworkers_y = plan.nty;
     else if (dist == 1)

@@ -18,7 +18,7 @@ struct EngineSpec {
     int A, B, K, NV, NU;
     int LX, LY, LV, LU;
     int WX, WY, RL, KBX;
-    int IW; // independent wavefronts (work items) per workgroup
+    int WZ; // wavefronts per workgroup that split one tile's rows and share the LDS bands
     int lds_bytes;
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
@@ -54,7 +54,7 @@ constexpr EngineSpec make_spec(const char *name) {
                       C::LY,  C::LV,
                       C::LU,  C::WX,
                       C::WY,  C::RL,
-                      C::KBX, C::IW,
+                      C::KBX, C::WZ,
                       C::LDS_BYTES,
                       C::NT,  &launch_engine<C>};
 }

@@ -223,6 +223,37 @@ def test_every_tile_specialisation(oracle):
                     check(got, oracle.n_to_m(left, right), True, f"tile {kw} {shape}")
 
 
+def test_every_compiled_specialisation_by_index(oracle):
+    """Runs every entry of the specialisation tables (all register tiles, lane layouts and the
+    ways wavefronts share a tile), unsplit and with the reduction split into atomically added
+    chunks, on shapes that span several staged bands and do not divide any tile."""
+    xc = load_package()
+    rng = np.random.default_rng(650)
+    for dtype in (np.float32, np.float64):
+        cases = []
+        for n_left, n_right, shape in [(3, 5, (19, 23)), (2, 3, (75, 45))]:
+            left = ints(rng, (n_left,) + shape, dtype)
+            right = ints(rng, (n_right,) + shape, dtype)
+            cases.append((n_left, n_right, shape, left, right, oracle.n_to_m(left, right, threads=4)))
+        index, names = 1, []
+        while True:
+            try:
+                for n_left, n_right, shape, left, right, exp in cases:
+                    for rows in (0, 20):
+                        kw = dict(specialisation=index, rows_per_thread=rows)
+                        got = xc.run("multimat_both_grouped", left, right, n_left * n_right, n_left=n_left, n_right=n_right,
+                                     params=xc.make_params(**kw))
+                        rec = xc.last_launch()
+                        check(got, exp, True, f"spec {index} {rec['kernel']} rows={rows} {shape}")
+                names.append(rec["kernel"])
+            except xc.XcorrError as e:
+                assert "does not exist" in e.message, e
+                break
+            index += 1
+        say(np.dtype(dtype).name, len(names), "specialisations:", " ".join(n.split("/")[1] for n in names))
+        assert len(names) >= 9
+
+
 def test_launch_record_and_errors():
     xc = load_package()
     rng = np.random.default_rng(700)
