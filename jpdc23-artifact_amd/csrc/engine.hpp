@@ -50,12 +50,12 @@ struct EngineArgs {
 };
 
 // WZ_ > 1: the WZ_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
-// matrices and split its left rows: a stage holds WZ_ (or a multiple) groups of G left rows, staged
-// by all threads together, and each wavefront sweeps its own groups. The wavefronts do the same
-// amount of work per stage, so the barriers around a stage cost little (wavefronts that own
-// different shift tiles skip different parts of a stage and wait for each other), the block tile
-// is as small as the wavefront tile (less work on partial overlaps), and the longest work item
-// of a launch is WZ_ times shorter. The partial sums are added through LDS before the tile is
+// matrices and split the reduction: a stage holds WZ_ (or a multiple) chunks of K columns, staged
+// by all threads together, and wavefront w sweeps the chunks kc = w (mod WZ_) over all rows of
+// the stage. The wavefronts do the same amount of work per stage, so the barriers around a stage
+// cost little (wavefronts that own different shift tiles skip different parts of a stage and
+// wait for each other), the block tile is as small as the wavefront tile (less work on partial
+// overlaps), and the longest work item of a launch is WZ_ times shorter. The partial sums are added through LDS before the tile is
 // written, or added atomically by each wavefront when the output is accumulated atomically anyway.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
           int RL_, int KBX_, int MINB_, int WZ_ = 1>
@@ -90,7 +90,7 @@ struct EngineCfg {
     static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
     static_assert(WZ == 1 || (WX == 1 && WY == 1 && A % WZ == 0), "row-splitting wavefronts share one wavefront tile");
-    static_assert((RL / (A_ + 1)) % WZ == 0, "every wavefront gets the same number of row groups per stage");
+    static_assert((KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
@@ -223,7 +223,7 @@ __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_l
     using vec = typename vec128<T>::type;
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK, G = C::G;
     constexpr int VW = C::VWIN_VECS * VK;
-    for (int kc = kc_lo; kc < kc_hi; ++kc) {
+    for (int kc = kc_lo; kc < kc_hi; kc += C::WZ) { // (kc_lo is this wavefront's first chunk)
         const T *vp = Vs_lane + kc * K + jj_lo * G * C::PV;
         const T *up = Us_lane + kc * K + jj_lo * G * C::PU;
         T ring[NU][G][K];
@@ -415,12 +415,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             if (first > 0) jj_lo = first / C::G;
             int h = last < 0 ? 0 : last / C::G + 1;
             if (h < jj_hi) jj_hi = h;
-            if (C::WZ > 1) {
-                // this wavefront's groups of the stage
-                constexpr int M = C::RL / C::G / C::WZ;
-                if (jj_lo < group * M) jj_lo = group * M;
-                if (jj_hi > (group + 1) * M) jj_hi = (group + 1) * M;
-            }
         }
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
             if (x0 == xr_lo && yl0 == clo)
@@ -464,6 +458,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                 int h = lim < 0 ? 0 : lim / K + 1;
                 if (h < kc_hi) kc_hi = h;
             }
+            if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
             if (jj_lo >= jj_hi) continue;
 
             compute_stage<C>(Vs_lane, Us_lane, acc, kc_lo, kc_hi, jj_lo, jj_hi);

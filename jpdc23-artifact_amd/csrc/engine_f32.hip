@@ -20,19 +20,19 @@ using R_2x2 = EngineCfg<float, 1, 8, 4, 2, 2, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 // several matrices per lane (the reference's left/right_matrices_per_thread), 2x2 wavefronts
 using G_48_n2 = EngineCfg<float, 4, 8, 4, 1, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
 using G_44_n22 = EngineCfg<float, 4, 4, 4, 2, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
-// grouped tiles: four wavefronts share one tile and its bands and take one group of rows each per
-// stage (WZ = 4). Lanes over shifts only ...
+// grouped tiles: four wavefronts share one tile and its bands and take every fourth chunk of columns of
+// a stage (WZ = 4). Lanes over shifts only ...
 using Z_84 = EngineCfg<float, 8, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
 using Z_88 = EngineCfg<float, 8, 8, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
 using Z_44 = EngineCfg<float, 4, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 20, 32, 4, 4>;
 // ... and lanes over right matrices (one_to_many, n_to_mn) or over pairs (n_to_m) of small matrices
 using Z_84_u4 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 4, 1, 4, 1, 1, 36, 16, 4, 4>;
 using Z_88_u4 = EngineCfg<float, 8, 8, 4, 1, 1, 4, 4, 1, 4, 1, 1, 36, 16, 4, 4>;
-using Z_84_u16 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 4, 4>;
-using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 4, 4>;
-using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
-using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
-using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 36, 8, 4, 4>;
+using Z_84_u16 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 1, 16, 1, 1, 18, 16, 4, 4>;
+using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 18, 16, 4, 4>;
+using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
+using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
+using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 18, 16, 4, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),

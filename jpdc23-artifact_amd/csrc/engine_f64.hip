@@ -10,29 +10,30 @@ namespace xcorr {
 // one output row per lane, 2x2 wavefronts over the shifts
 using R_1x1 = EngineCfg<double, 1, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
 using R_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
-// grouped tiles: four wavefronts share one tile and its bands and take one group of rows each per stage
+// grouped tiles: four wavefronts share one tile and its bands and take every fourth chunk of columns of a stage
 using Z_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 2, 4>;
-using Z_84 = EngineCfg<double, 8, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 4, 4>;
 using Z_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 20, 16, 4, 4>;
 using Z_88_u4 = EngineCfg<double, 8, 8, 2, 1, 1, 4, 4, 1, 4, 1, 1, 36, 8, 2, 4>;
-using Z_84_u4 = EngineCfg<double, 8, 4, 2, 1, 1, 4, 4, 1, 4, 1, 1, 36, 8, 4, 4>;
 using Z_88_u16 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 1, 16, 1, 1, 36, 8, 2, 4>;
 using Z_88_v4u4 = EngineCfg<double, 8, 8, 2, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 2, 4>;
-using Z_84_v4u4 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 4, 4>;
 using Z_88_v8u8 = EngineCfg<double, 8, 8, 2, 1, 1, 1, 1, 8, 8, 1, 1, 36, 8, 2, 4>;
+// 8x4 tiles of doubles fit 168 VGPRs: three wavefronts per SIMD
+using Y_84_u4 = EngineCfg<double, 8, 4, 2, 1, 1, 4, 4, 1, 4, 1, 1, 36, 8, 3, 4>;
+using Y_84_v4u4 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 2, 4, 4, 1, 1, 36, 8, 3, 4>;
+using Y_84 = EngineCfg<double, 8, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 3, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
     make_spec<R_2x2>("f64_a1b4_l2r2"),
     make_spec<Z_88>("f64_a8b8"),
-    make_spec<Z_84>("f64_a8b4"),
     make_spec<Z_44>("f64_a4b4"),
     make_spec<Z_88_u4>("f64_a8b8_lr4"),
-    make_spec<Z_84_u4>("f64_a8b4_lr4"),
     make_spec<Z_88_u16>("f64_a8b8_lr16"),
     make_spec<Z_88_v4u4>("f64_a8b8_ll4lr4"),
-    make_spec<Z_84_v4u4>("f64_a8b4_ll4lr4"),
     make_spec<Z_88_v8u8>("f64_a8b8_ll8lr8"),
+    make_spec<Y_84_u4>("f64_a8b4_lr4"),
+    make_spec<Y_84_v4u4>("f64_a8b4_ll4lr4"),
+    make_spec<Y_84>("f64_a8b4"),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {

@@ -35,8 +35,9 @@ static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)
 //   * lanes idling over matrices that do not exist;
 //   * the issue rate of the tile: one-row tiles lose issue slots to LDS reads (a read plus the
 //     wait that guards it displace about nine fp32 FMA slots, half as many fp64 ones); among
-//     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower;
-//   * lanes laid over more than four matrices stage many small bands: +12.5 % per doubling.
+//     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower (fp64: 8x8 5 % slower);
+//   * lanes laid over matrices stage one band per matrix, and a right band carries a halo of
+//     TYW-1 rows: +3.5 % per extra right matrix, +2 % per extra left matrix.
 // Hints scale the cost so the nearest specialisation wins without excluding the others.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
@@ -51,12 +52,11 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
         double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
         cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
     } else if (s.A == 8 && s.B == 8) {
-        cost *= s.elem_bytes == 4 ? 1.08 : 1.0;
+        cost *= s.elem_bytes == 4 ? 1.08 : 1.05;
     } else if (s.A == 4 && s.B == 4) {
-        cost *= 1.08;
+        cost *= s.elem_bytes == 4 ? 1.08 : 1.0;
     }
-    double matrix_lanes = std::log2((double)(s.LV * s.LU));
-    if (matrix_lanes > 2) cost *= 1.0 + 0.125 * (matrix_lanes - 2);
+    cost *= 1.0 + 0.035 * (s.LU - 1) + 0.02 * (s.LV - 1);
     if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
     if (s.WX * s.WY * s.WZ < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
     if (s.A > 1 && s.WZ == 1) cost *= 1.1; // shift-tiled blocks wait at the barriers of partial stages
@@ -131,16 +131,20 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         plan.atomic = 1;
         plan.zero_fill = false;
     } else {
-        // Few tiles: cut the reduction into chunks of whole staged bands (at least two per item)
+        // Few tiles, or long ones: cut the reduction into chunks of whole staged bands
         // until the launch has about 64 work items per CU; finer items even out the last wave of
         // blocks, coarser ones save atomics (measured on 1024x1024: 16 per CU is 10 % slower).
         // Lanes laid over matrices write one result matrix per lane: their atomics would not
         // coalesce, so such tiles are never split by the planner itself.
         const bool split_ok = rq.may_split && best->LV * best->LU == 1;
-        if (rc <= 0 && split_ok && tiles < 24L * device_cus()) {
+        const int k_most = 8; // longest item: eight staged bands (2048x2048 unsplit is 20 % slower than in chunks)
+        if (rc <= 0 && split_ok && (tiles < 24L * device_cus() || rq.H > k_most * best->RL)) {
             const long target = 64L * device_cus();
             const long per_tile_column = (long)plan.ntx * plan.nvg * plan.nug;
-            for (int k = rq.H / best->RL; k >= 2; --k) {
+            // (an item of a single band only when two-band items would leave CUs without work)
+            const int k_min = per_tile_column * count_chunks(*best, rq.H, plan.nty, 2 * best->RL, nullptr) < 2L * device_cus() ? 1 : 2;
+            int k = rq.H / best->RL < k_most ? rq.H / best->RL : k_most;
+            for (; k >= k_min; --k) {
                 rc = k * best->RL;
                 if (per_tile_column * count_chunks(*best, rq.H, plan.nty, rc, nullptr) >= target) break;
             }
