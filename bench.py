@@ -22,9 +22,9 @@ from __graft_entry__ import load_oracle, load_package  # noqa: E402
 # MI355X published vector peaks (TFLOP/s)
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
-# by the library's copy kernel (figures and commands: profiles/engine_f32_a8b8_one_to_one_1024.md).
+# by the library's copy kernel (figures and commands: profiles/engine_f32_a8b4_one_to_one_1024.md).
 # Only the default workload with default parameters has been measured.
-MEASURED_TRAFFIC_BYTES = {"C2": 0.812e9 + 1.495e9}
+MEASURED_TRAFFIC_BYTES = {"C2": 2.57e9 + 2.60e9}
 
 
 def cpu_baseline(oracle, cfg, left, right, budget_s=15.0):
@@ -206,6 +206,17 @@ def main():
             "max_abs": float(f"{e.max_abs:.3e}"),
             "max_rel": float(f"{e.max_rel:.3e}"),
         }
+        if dtype == np.float32:
+            # the host loop adds every overlap one product at a time in fp32 and drifts from the exact
+            # sum on long overlaps; the same loop with an fp64 accumulator tells the two apart
+            mid = (lo + hi) // 2
+            lo64, hi64 = max(lo, mid - 8), min(hi, mid + 8)
+            exact = oracle.cross_corr(left[0], right[0], threads=base["cores"], row_begin=lo64, row_end=hi64, acc64=True)
+            e64 = oracle.errors(got[0][lo64:hi64], exact[lo64:hi64])
+            o64 = oracle.errors(band[lo64:hi64], exact[lo64:hi64])
+            result["parity"]["rows_checked_with_fp64_accumulator"] = [lo64, hi64]
+            result["parity"]["rel_frobenius_vs_fp64_accumulated"] = float(f"{e64.rel_frobenius:.3e}")
+            result["parity"]["oracle_fp32_vs_fp64_accumulated"] = float(f"{o64.rel_frobenius:.3e}")
     print(json.dumps(result))
 
 
