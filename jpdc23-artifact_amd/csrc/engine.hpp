@@ -57,13 +57,16 @@ struct EngineArgs {
 // wait for each other), the block tile is as small as the wavefront tile (less work on partial
 // overlaps), and the longest work item of a launch is WZ_ times shorter. The partial sums are added through LDS before the tile is
 // written, or added atomically by each wavefront when the output is accumulated atomically anyway.
+// DB_ = 1: two sets of LDS bands. While the wavefronts sweep one, the next stage is copied into the
+// other by the memory pipeline itself (loads that write LDS directly, no registers, no waiting
+// wavefront), and one barrier per stage is enough.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
-          int RL_, int KBX_, int MINB_, int WZ_ = 1>
+          int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0>
 struct EngineCfg {
     using value_type = T;
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
-    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_;
+    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_;
     static constexpr int VK = 16 / (int)sizeof(T); // elements per 128-bit LDS access
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
@@ -87,7 +90,8 @@ struct EngineCfg {
     // in-block reduction: one output row of the tile per wavefront and pass, [owner][source][lane][RED_ROW]
     static constexpr int RED_ROW = NV * NU * B;
     static constexpr int RED_ELEMS = WZ > 1 ? WZ * WZ * 64 * RED_ROW : 0;
-    static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
+    static constexpr int LDS_BUFFERS = DB ? 2 : 1;
+    static constexpr int LDS_BYTES = (LDS_ELEMS * LDS_BUFFERS > RED_ELEMS ? LDS_ELEMS * LDS_BUFFERS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
     static_assert(WZ == 1 || (WX == 1 && WY == 1 && A % WZ == 0), "row-splitting wavefronts share one wavefront tile");
     static_assert((KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
@@ -121,7 +125,9 @@ struct PhaseClock {
     }
     __device__ __forceinline__ void lap(int phase) {
         long long now = (long long)clock64();
-        acc[phase] += now - t;
+#pragma unroll
+        for (int i = 0; i < PH_COUNT; ++i) // (no dynamic indexing: the table stays in registers)
+            if (i == phase) acc[i] += now - t;
         t = now;
     }
     __device__ __forceinline__ void flush() {
@@ -204,8 +210,60 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
     }
 }
 
+// Lane i of the wavefront copies the 16 bytes at its own global address to LDS byte address
+// lds_base + 16 * i, without passing through registers; completion is counted by vmcnt. The
+// compiler does not know that this writes LDS: callers wait (dma_wait) and pass a barrier before
+// anything reads the destination.
+__device__ __forceinline__ void dma16(const void *gptr, unsigned lds_base) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_base) : "memory", "m0");
+}
+__device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+
+// stage_bands with the copies done by dma16: pieces that lie fully inside the matrices are copied
+// asynchronously, pieces outside are zeroed and pieces that straddle a matrix edge are assembled
+// element by element with ordinary stores. The image is addressed linearly in 128-bit pieces
+// (band * BAND/VK + row * PITCH/VK + column piece), which is what makes the 64 pieces of one
+// wavefront-wide copy contiguous in LDS.
+template <class C, int NB, int ROWS, int PITCH, int BAND>
+__device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride,
+                                                  int W, int nbands, int row_lo, int row_hi, int row0, int col0, int col_lo,
+                                                  int col_hi, int tid) {
+    using T = typename C::value_type;
+    using vec = typename vec128<T>::type;
+    constexpr int VK = C::VK, PP = PITCH / VK, BANDP = BAND / VK, TOTP = NB * BANDP;
+    constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
+    static_assert(PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
+    // LDS byte address of the piece of lane 0 of this wavefront in iteration 0
+    const unsigned wave_base =
+        __builtin_amdgcn_readfirstlane((unsigned)(size_t)lds) + (unsigned)__builtin_amdgcn_readfirstlane(tid & ~63) * 16u;
+#pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+        const int p = tid + it * C::NT;
+        const int band = p / BANDP, q = p % BANDP, row = q / PP, col = (q % PP) * VK;
+        if (p < TOTP && row < ROWS) {
+            const bool inside = band < nbands && row >= row_lo && row < row_hi;
+            const T *gp = src + (size_t)band * mat_stride + (ptrdiff_t)(row0 + row) * W + (ptrdiff_t)(col0 + col);
+            if (inside && col >= col_lo && col + VK <= col_hi) {
+                dma16(gp, wave_base + (unsigned)(it * C::NT) * 16u);
+            } else {
+                // zero the piece, then patch in the elements of a piece that straddles an edge (the
+                // patch is kept apart from the zeroing so that only it waits for its loads)
+                vec zero;
+#pragma unroll
+                for (int e = 0; e < VK; ++e) zero[e] = T(0);
+                *reinterpret_cast<vec *>(lds + (size_t)p * VK) = zero;
+                if (inside && col + VK > col_lo && col < col_hi) {
+#pragma unroll
+                    for (int e = 0; e < VK; ++e)
+                        if (col + e >= col_lo && col + e < col_hi) lds[(size_t)p * VK + e] = gp[e];
+                }
+            }
+        }
+    }
+}
+
 // Inner loops of one stage for one lane: for every K-column chunk kc in [kc_lo, kc_hi) sweep
-// the groups of G staged left rows jj in [jj_lo, jj_hi).
+// the groups of G staged left rows jj in [jj_lo, jj_hi) and `tail` (< G) more rows after them.
 //
 // Register plan per lane: NV*NU*A*B accumulators, a ring of G = A+1 right rows (row j in
 // slot j mod G, so the row of the next step is fetched while the current step still uses
@@ -218,7 +276,7 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
 template <class C>
 __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
                                               typename C::value_type (&acc)[C::NV][C::NU][C::A][C::B], int kc_lo,
-                                              int kc_hi, int jj_lo, int jj_hi) {
+                                              int kc_hi, int jj_lo, int jj_hi, int tail) {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK, G = C::G;
@@ -247,10 +305,11 @@ __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_l
 #pragma unroll
                 for (int e = 0; e < VK; ++e) vw[i][q * VK + e] = r[e];
             }
-#pragma unroll 1
-        for (int jj = jj_lo; jj < jj_hi; ++jj) {
+        // `tail` left rows follow the full groups: the last group stops after them
+        auto group = [&](int steps) __attribute__((always_inline)) {
 #pragma unroll
             for (int s = 0; s < G; ++s) {
+                if (s > 0 && s >= steps) break;
                 // right row s+1 (at s = G-1: the first row of the next group, or the spare
                 // row the bands keep at their end)
 #pragma unroll
@@ -291,9 +350,14 @@ __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_l
                     }
                 }
             }
+        };
+#pragma unroll 1
+        for (int jj = jj_lo; jj < jj_hi; ++jj) {
+            group(G);
             vp += G * C::PV;
             up += G * C::PU;
         }
+        if (tail > 0) group(tail);
     }
 }
 
@@ -404,64 +468,104 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
 
     const size_t HW = (size_t)W * H;
 
-    for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
-        // groups of G left rows of this stage that can overlap this wavefront's y shifts
-        int jj_lo = 0, jj_hi = C::RL / C::G;
+    // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner).
+    const int nxs = xr_hi > xr_lo ? (xr_hi - xr_lo + C::KBX - 1) / C::KBX : 0;
+    const int nstages = nxs * ((chi - clo + C::RL - 1) / C::RL);
+
+    // fills one set of bands with the stage at left rows [yl0, yl0+RL), right columns [x0, x0+KBX)
+    auto stage = [&](T *buf, int yl0, int x0) __attribute__((always_inline)) {
+        // left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col
+        const int xbase = x0 + sxb;
+        const int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
+        const int nbv = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
+        const int vc_lo = xbase < 0 ? -xbase : 0;
+        const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
+        // right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col
+        const int yr0 = yl0 - syb - C::TYB + 1;
+        const int nbu = u_limit - u_first < C::NUB ? u_limit - u_first : C::NUB;
+        const int ur_lo = yr0 < 0 ? -yr0 : 0;
+        const int ur_hi = H - yr0 < C::RU + 1 ? H - yr0 : C::RU + 1;
+        const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
+        T *ubuf = buf + C::NVB * C::VBAND;
+        if constexpr (C::DB) {
+            stage_bands_async<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, W, nbv, 0, rows_ok, yl0, xbase,
+                                                                     vc_lo, vc_hi, tid);
+            stage_bands_async<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, W, nbu, ur_lo, ur_hi, yr0, x0,
+                                                                     0, uc_hi, tid);
+        } else {
+            stage_bands<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, W, nbv, 0, rows_ok, yl0, xbase, vc_lo,
+                                                               vc_hi, tid);
+            stage_bands<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, W, nbu, ur_lo, ur_hi, yr0, x0, 0,
+                                                               uc_hi, tid);
+        }
+    };
+    // this wavefront's part of a staged stage
+    auto compute = [&](int buf_offset, int yl0, int x0) __attribute__((always_inline)) {
+        // groups of G left rows of this stage that can overlap this wavefront's y shifts:
+        // rows yl in [syw, syw + TYW - 1 + H - 1] and yl < chi
+        int jj_lo = 0, jj_hi = C::RL / C::G, tail = 0;
         {
-            // rows yl in [syw, syw + TYW - 1 + H - 1] and yl < chi
-            int first = syw - yl0;                     // first useful row index j
-            int last = syw + C::TYW + H - 2 - yl0;     // last useful row index j
+            int first = syw - yl0;                 // first useful row index j
+            int last = syw + C::TYW + H - 2 - yl0; // last useful row index j
             if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
             if (first > 0) jj_lo = first / C::G;
-            int h = last < 0 ? 0 : last / C::G + 1;
-            if (h < jj_hi) jj_hi = h;
+            const int rows = last < 0 ? 0 : last + 1; // useful rows from row 0 of the stage
+            if (rows < C::RL) {
+                jj_hi = rows / C::G;
+                tail = rows % C::G;
+            }
         }
-        for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
-            if (x0 == xr_lo && yl0 == clo)
-                pc.lap(PH_SETUP);
-            else
-                pc.lap(PH_COMPUTE);
-            __syncthreads(); // everyone is done reading the previous stage
-            pc.lap(PH_WAIT_SIBLINGS);
-            // ---- stage the left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col ----
-            {
-                const int xbase = x0 + sxb;
-                int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
-                int nb = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
-                int c_lo = xbase < 0 ? -xbase : 0;
-                int c_hi = W - xbase < C::PV ? W - xbase : C::PV;
-                stage_bands<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(Vs, g.V + (size_t)v_first * HW, HW, W, nb, 0, rows_ok, yl0, xbase, c_lo,
-                                                                   c_hi, tid);
-            }
-            // ---- stage the right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col ----
-            {
-                const int yr0 = yl0 - syb - C::TYB + 1;
-                int nb = u_limit - u_first < C::NUB ? u_limit - u_first : C::NUB;
-                int r_lo = yr0 < 0 ? -yr0 : 0;
-                int r_hi = H - yr0 < C::RU + 1 ? H - yr0 : C::RU + 1;
-                int c_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
-                stage_bands<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(Us, g.U + (size_t)u_first * HW, HW, W, nb, r_lo, r_hi, yr0, x0, 0, c_hi,
-                                                                   tid);
-            }
-            pc.lap(PH_STAGING);
-            __syncthreads();
+        // K-column chunks of this stage that overlap this wavefront's x shifts: need
+        // (x0 + kc*K + K-1) + (sxw + TXW-1) >= 0 and (x0 + kc*K) + sxw <= W-1 and x0 + kc*K < W
+        int kc_lo = 0, kc_hi = C::KBX / K;
+        {
+            int need = -(sxw + C::TXW - 1) - (K - 1) - x0;
+            if (need > 0) kc_lo = (need + K - 1) / K;
+            int lim = W - 1 - sxw - x0;
+            if (W - 1 - x0 < lim) lim = W - 1 - x0;
+            int h = lim < 0 ? 0 : lim / K + 1;
+            if (h < kc_hi) kc_hi = h;
+        }
+        if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
+        if (jj_lo < jj_hi || (jj_lo == jj_hi && tail > 0))
+            compute_stage<C>(Vs_lane + buf_offset, Us_lane + buf_offset, acc, kc_lo, kc_hi, jj_lo, jj_hi, tail);
+    };
+
+    if constexpr (C::DB) {
+        // stage s+1 is copied into one set of bands while stage s is swept in the other
+        if (nstages > 0) stage(Vs, clo, xr_lo);
+        int yl0 = clo, x0 = xr_lo; // stage being computed
+        for (int st = 0; st < nstages; ++st) {
+            pc.lap(st == 0 ? PH_SETUP : PH_COMPUTE);
+            dma_wait();
+            __syncthreads(); // stage st has landed for everyone, and everyone is done with stage st-1
             pc.lap(PH_WAIT_STAGED);
-
-            // ---- K-column chunks of this stage that overlap this wavefront's x shifts ----
-            int kc_lo = 0, kc_hi = C::KBX / K;
-            {
-                // need (x0 + kc*K + K-1) + (sxw + TXW-1) >= 0 and (x0 + kc*K) + sxw <= W-1 and x0 + kc*K < W
-                int need = -(sxw + C::TXW - 1) - (K - 1) - x0;
-                if (need > 0) kc_lo = (need + K - 1) / K;
-                int lim = W - 1 - sxw - x0;
-                if (W - 1 - x0 < lim) lim = W - 1 - x0;
-                int h = lim < 0 ? 0 : lim / K + 1;
-                if (h < kc_hi) kc_hi = h;
+            int yl1 = yl0, x1 = x0 + C::KBX;
+            if (x1 >= xr_hi) {
+                x1 = xr_lo;
+                yl1 += C::RL;
             }
-            if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
-            if (jj_lo >= jj_hi) continue;
-
-            compute_stage<C>(Vs_lane, Us_lane, acc, kc_lo, kc_hi, jj_lo, jj_hi);
+            const int cur = (st & 1) * C::LDS_ELEMS;
+            if (st + 1 < nstages) stage(Vs + (C::LDS_ELEMS - cur), yl1, x1);
+            pc.lap(PH_STAGING);
+            compute(cur, yl0, x0);
+            yl0 = yl1;
+            x0 = x1;
+        }
+    } else {
+        bool first_stage = true;
+        for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
+            for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
+                pc.lap(first_stage ? PH_SETUP : PH_COMPUTE);
+                first_stage = false;
+                __syncthreads(); // everyone is done reading the previous stage
+                pc.lap(PH_WAIT_SIBLINGS);
+                stage(Vs, yl0, x0);
+                pc.lap(PH_STAGING);
+                __syncthreads();
+                pc.lap(PH_WAIT_STAGED);
+                compute(0, yl0, x0);
+            }
         }
     }
 

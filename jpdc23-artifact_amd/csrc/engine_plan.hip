@@ -37,7 +37,7 @@ static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)
 //     wait that guards it displace about nine fp32 FMA slots, half as many fp64 ones); among
 //     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower (fp64: 8x8 5 % slower);
 //   * lanes laid over matrices stage one band per matrix, and a right band carries a halo of
-//     TYW-1 rows: +3.5 % per extra right matrix, +2 % per extra left matrix.
+//     TYW-1 rows: +2.8 % per extra right matrix, +2 % per extra left matrix.
 // Hints scale the cost so the nearest specialisation wins without excluding the others.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
@@ -56,7 +56,7 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     } else if (s.A == 4 && s.B == 4) {
         cost *= s.elem_bytes == 4 ? 1.08 : 1.0;
     }
-    cost *= 1.0 + 0.035 * (s.LU - 1) + 0.02 * (s.LV - 1);
+    cost *= 1.0 + 0.028 * (s.LU - 1) + 0.02 * (s.LV - 1);
     if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
     if (s.WX * s.WY * s.WZ < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
     if (s.A > 1 && s.WZ == 1) cost *= 1.1; // shift-tiled blocks wait at the barriers of partial stages
