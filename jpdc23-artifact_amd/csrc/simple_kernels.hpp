@@ -190,11 +190,29 @@ __global__ __launch_bounds__(1024) void warp_per_overlap_kernel(const T *__restr
     const int ow = xr_hi - xr_lo, oh = yr_hi - yr_lo;
     T sum = T(0);
     if (VARIANT == 1) {
-        for (int yr = yr_lo; yr < yr_hi; ++yr) {
-            const T *rrow = right + (size_t)yr * W;
-            const T *lrow = left + (size_t)(yr + sy) * W + sx;
-            for (int xr = xr_lo + lane; xr < xr_hi; xr += 64) sum += lrow[xr] * rrow[xr];
+        // columns outer (one pass up to 64 columns), rows inner and unrolled eight times with
+        // independent partial sums: sixteen loads are in flight per lane instead of two, which is
+        // what a wavefront that owns a single short reduction needs to hide the cache latency
+        T part_sum[8];
+#pragma unroll
+        for (int r = 0; r < 8; ++r) part_sum[r] = T(0);
+        for (int xr = xr_lo + lane; xr < xr_hi; xr += 64) {
+            const T *rp = right + (size_t)yr_lo * W + xr;
+            const T *lp = left + (size_t)(yr_lo + sy) * W + (sx + xr);
+            int yr = yr_lo;
+            for (; yr + 8 <= yr_hi; yr += 8) {
+#pragma unroll
+                for (int r = 0; r < 8; ++r) part_sum[r] += lp[(size_t)r * W] * rp[(size_t)r * W];
+                lp += (size_t)8 * W;
+                rp += (size_t)8 * W;
+            }
+            for (; yr < yr_hi; ++yr) {
+                part_sum[0] += lp[0] * rp[0];
+                lp += W;
+                rp += W;
+            }
         }
+        sum = ((part_sum[0] + part_sum[1]) + (part_sum[2] + part_sum[3])) + ((part_sum[4] + part_sum[5]) + (part_sum[6] + part_sum[7]));
     } else if (oh > 0 && ow > 0) {
         const unsigned total = (unsigned)ow * (unsigned)oh;
         for (unsigned i = lane; i < total; i += 64) {
