@@ -55,8 +55,9 @@ struct EngineArgs {
 // the stage. The wavefronts do the same amount of work per stage, so the barriers around a stage
 // cost little (wavefronts that own different shift tiles skip different parts of a stage and
 // wait for each other), the block tile is as small as the wavefront tile (less work on partial
-// overlaps), and the longest work item of a launch is WZ_ times shorter. The partial sums are added through LDS before the tile is
-// written, or added atomically by each wavefront when the output is accumulated atomically anyway.
+// overlaps), and the longest work item of a launch is WZ_ times shorter. The partial sums are
+// added through LDS before the tile is written (or atomically added, once per block, when the
+// reduction is also split over work items).
 // DB_ = 1: two sets of LDS bands. While the wavefronts sweep one, the next stage is copied into the
 // other by the memory pipeline itself (loads that write LDS directly, no registers, no waiting
 // wavefront), and one barrier per stage is enough.
@@ -575,7 +576,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const size_t out_area = (size_t)Sx * Sy;
     const int ox0 = sxw + lx * B + (W - 1);
     const int oy0 = syw + ly * A + (H - 1);
-    if (C::WZ > 1 && !g.atomic) {
+    if (C::WZ > 1) {
         // Add the partial tiles of the WZ wavefronts. In pass q wavefront w ends up with the
         // sums of tile row q*WZ + w: everyone deposits rows q*WZ .. q*WZ+WZ-1, then reads back
         // all WZ versions of its own row (in wavefront order, so the result is deterministic).
@@ -643,7 +644,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         pc.flush();
         return;
     }
-    // (row-splitting wavefronts of an atomically accumulated tile add their partial sums directly)
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
         const int v = v_first + lv * NV + i;

@@ -131,21 +131,26 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         plan.atomic = 1;
         plan.zero_fill = false;
     } else {
-        // Few tiles, or long ones: cut the reduction into chunks of whole staged bands
-        // until the launch has about 64 work items per CU; finer items even out the last wave of
-        // blocks, coarser ones save atomics (measured on 1024x1024: 16 per CU is 10 % slower).
-        // Lanes laid over matrices write one result matrix per lane: their atomics would not
-        // coalesce, so such tiles are never split by the planner itself.
+        // Few tiles, or long ones: cut the reduction over left rows into chunks (whole groups of
+        // G = A+1 rows, the granule of the inner loop) until the launch has about 128 work items
+        // per CU. Finer items even out the last wave of blocks and cost little, because the four
+        // wavefronts of a block add their partial tiles in LDS before the atomic adds (1024x1024:
+        // flat between 18 and 54 rows, 3 % slower at 72, 6 % at 144; 2048x2048 unsplit 20 % slower).
+        // Items shorter than 20 rows only pay for tiny problems that would otherwise leave CUs
+        // without work. Lanes laid over matrices write one result matrix per lane: their
+        // atomics would not coalesce, so such tiles are never split by the planner itself.
         const bool split_ok = rq.may_split && best->LV * best->LU == 1;
-        const int k_most = 8; // longest item: eight staged bands (2048x2048 unsplit is 20 % slower than in chunks)
-        if (rc <= 0 && split_ok && (tiles < 24L * device_cus() || rq.H > k_most * best->RL)) {
-            const long target = 64L * device_cus();
+        const int G = best->A + 1;
+        const int rc_most = 4 * best->RL;
+        if (rc <= 0 && split_ok && (tiles < 48L * device_cus() || rq.H > rc_most)) {
+            const long target = 128L * device_cus();
             const long per_tile_column = (long)plan.ntx * plan.nvg * plan.nug;
-            // (an item of a single band only when two-band items would leave CUs without work)
-            const int k_min = per_tile_column * count_chunks(*best, rq.H, plan.nty, 2 * best->RL, nullptr) < 2L * device_cus() ? 1 : 2;
-            int k = rq.H / best->RL < k_most ? rq.H / best->RL : k_most;
+            // shortest item: 20 rows, or 9 when that leaves CUs without work (rounded up to whole groups)
+            const int k_normal = ceil_div(20, G), k_tiny = ceil_div(9, G);
+            const int k_min = per_tile_column * count_chunks(*best, rq.H, plan.nty, k_normal * G, nullptr) < 2L * device_cus() ? k_tiny : k_normal;
+            int k = (rq.H < rc_most ? rq.H : rc_most) / G;
             for (; k >= k_min; --k) {
-                rc = k * best->RL;
+                rc = k * G;
                 if (per_tile_column * count_chunks(*best, rq.H, plan.nty, rc, nullptr) >= target) break;
             }
             if (rc <= 0) rc = rq.H;
