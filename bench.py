@@ -24,7 +24,7 @@ PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
 # by the library's copy kernel (figures and commands: profiles/engine_f32_a8b4_one_to_one_1024.md).
 # Only the default workload with default parameters has been measured.
-MEASURED_TRAFFIC_BYTES = {"C2": 2.57e9 + 2.60e9}
+MEASURED_TRAFFIC_BYTES = {"C2": 3.02e9 + 1.64e9}
 
 
 def cpu_baseline(oracle, cfg, left, right, budget_s=15.0):
