@@ -77,6 +77,13 @@ typedef struct xcorr_params {
     unsigned lanes_x;                        /* lanes of a wavefront laid along x shifts (power of two) */
     unsigned lanes_y;                        /* lanes laid along y shifts; the rest are laid over matrices */
     unsigned specialisation;                 /* 1-based index into the compiled tile list of the dtype (tuning sweeps) */
+    /* warp-per-overlap through LDS (one_to_one.hpp:568-572) and block-per-overlap (one_to_one.hpp:649) */
+    unsigned shared_mem_row_size;            /* columns staged per pass; this build always stages 64 (one per lane) */
+    unsigned shared_mem_rows;                /* right rows staged per pass; 0 = shifts_per_thread_block, smaller is an error */
+    unsigned right_matrices_per_block;       /* 0 = 1; <= 8 */
+    unsigned strided_load;                   /* load pattern of the reference's staging; no effect here */
+    unsigned column_group_per_block;         /* 1: one block per group of 64 columns, sums added atomically (caller zeroes `out`) */
+    unsigned block_size;                     /* block-per-overlap: threads per block, 0 = 128, <= 1024 */
     unsigned reserved[2];
 } xcorr_params;
 
@@ -164,6 +171,25 @@ int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out
                                const xcorr_params *p, void *stream);
 int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                const xcorr_params *p, void *stream);
+
+/* Warp-per-overlap through LDS: the wavefronts of a block own consecutive y shifts of
+ * one x shift and share staged row chunks of the left matrix and of up to eight right
+ * matrices. Replaces run_ccn_warp_per_shift_shared_mem (kernels.cuh:144-161). One left
+ * matrix against `n_right` right matrices, result i belongs to right matrix i. Uses
+ * p->shifts_per_thread_block (<= 32; at most 16 wavefronts fit a block),
+ * p->shared_mem_rows, p->right_matrices_per_block and p->column_group_per_block
+ * (then the caller zeroes `out` first, as one_to_one.hpp:600-605). */
+int xcorr_warp_per_overlap_lds_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                   unsigned n_right, const xcorr_params *p, void *stream);
+int xcorr_warp_per_overlap_lds_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                   unsigned n_right, const xcorr_params *p, void *stream);
+
+/* Block-per-overlap: all wavefronts of a block reduce one shift together.
+ * Replaces run_ccn_block_per_shift (kernels.cuh:197-205). One pair. Uses p->block_size. */
+int xcorr_block_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                const xcorr_params *p, void *stream);
+int xcorr_block_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                const xcorr_params *p, void *stream);
 
 /* Sliding-window base: every lane owns adjacent x shifts of one output row.
  * Replaces run_ccn_shuffle (kernels.cuh:65-73). One pair. Uses p->warps_per_thread_block. */

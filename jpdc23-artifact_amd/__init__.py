@@ -44,6 +44,12 @@ class Params(ctypes.Structure):
         ("lanes_x", ctypes.c_uint),
         ("lanes_y", ctypes.c_uint),
         ("specialisation", ctypes.c_uint),
+        ("shared_mem_row_size", ctypes.c_uint),
+        ("shared_mem_rows", ctypes.c_uint),
+        ("right_matrices_per_block", ctypes.c_uint),
+        ("strided_load", ctypes.c_uint),
+        ("column_group_per_block", ctypes.c_uint),
+        ("block_size", ctypes.c_uint),
         ("reserved", ctypes.c_uint * 2),
     ]
 
@@ -223,6 +229,8 @@ def make_params(**kw):
 FAMILIES = {
     "overlap_wise": ("xcorr_overlap_wise", "batch", False),
     "warp_per_overlap": ("xcorr_warp_per_overlap", "pair", None),
+    "warp_per_overlap_lds": ("xcorr_warp_per_overlap_lds", "right", None),
+    "block_per_overlap": ("xcorr_block_per_overlap", "pair", False),
     "shuffle": ("xcorr_shuffle", "pair", False),
     "split_row": ("xcorr_split_row", "pair", True),
     "grouped_overlap": ("xcorr_grouped_overlap", "pair", False),
@@ -267,6 +275,8 @@ def needs_zeroed_output(family, params):
         return params is not None and params.warp_per_overlap_variant == 2
     if family == "multimat_right":
         return params is not None and params.rows_per_thread > 0
+    if family == "warp_per_overlap_lds":
+        return params is not None and params.column_group_per_block != 0
     return False
 
 

@@ -7,6 +7,11 @@
 //                     partial sums are combined with DPP row operations (no LDS, no
 //                     ds_bpermute), replacing the 32-lane cg::reduce of
 //                     naive_warp_per_shift.cu:21-244.
+// warp-per-overlap, LDS : the wavefronts of a block own consecutive y shifts of one x shift
+//                     and share row chunks of the right matrices and of the left matrix
+//                     staged in LDS (naive_warp_per_shift_shared_mem.cu:160-420).
+// block-per-overlap : all wavefronts of a block reduce one shift together
+//                     (naive_block_per_shift.cu:17-97).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -280,6 +285,209 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
     rec.rows_per_worker = variant == 2 ? max_rows : rows;
     rec.distribution_type = variant == 2 ? dist : XCORR_DIST_NONE;
     rec.uses_atomics = variant == 2;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+// ------------------------------------------------------------------ warp-per-overlap through LDS
+// Block = NW wavefronts; wavefront w owns shift (sx, sy0 + w) for NR right matrices of one
+// group. Per pass the block stages `SR` rows x 64 columns of each right matrix and the
+// SR + NW - 1 left rows those shifts pair them with (zero outside the matrices, so the sweep
+// has no bounds checks), then every wavefront multiplies its own diagonal of row pairs:
+// lane = column, one LDS read of the left row and NR reads of right rows per NR FMAs.
+// gridDim.z > 1: block z owns the 64-column group z only and adds its sums atomically.
+template <typename T, int NR>
+__global__ __launch_bounds__(1024) void warp_per_overlap_lds_kernel(const T *__restrict__ left, const T *__restrict__ right,
+                                                                     T *__restrict__ out, int W, int H, int n_right, int SR) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char wpo_smem[];
+    T *Ls = reinterpret_cast<T *>(wpo_smem);                      // [SR + NW - 1][64]
+    const int NW = blockDim.y;
+    T *Rs = Ls + (size_t)(SR + NW - 1) * 64;                       // [NR][SR][64]
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
+    const int lane = threadIdx.x, w = threadIdx.y;
+    const int tid = w * 64 + lane, nthreads = NW * 64;
+    const int ox = blockIdx.x % Sx, group = blockIdx.x / Sx;
+    const int sx = ox - (W - 1);
+    const int sy0 = (int)blockIdx.y * NW - (H - 1);
+    const int oy = (int)blockIdx.y * NW + w;
+    const int m0 = group * NR;
+    const int nr = n_right - m0 < NR ? n_right - m0 : NR;
+    // overlap of the block in right-matrix coordinates: columns of this x shift, rows of any of its y shifts
+    int xr_lo = sx < 0 ? -sx : 0, xr_hi = W - sx < W ? W - sx : W;
+    if (gridDim.z > 1) {
+        xr_lo += (int)blockIdx.z * 64;
+        if (xr_lo + 64 < xr_hi) xr_hi = xr_lo + 64;
+        if (xr_lo >= xr_hi) return;
+    }
+    const int sy_max = sy0 + NW - 1;
+    const int yr_lo = sy_max < 0 ? -sy_max : 0;
+    const int yr_hi = H - sy0 < H ? H - sy0 : H;
+    T sum[NR];
+#pragma unroll
+    for (int m = 0; m < NR; ++m) sum[m] = T(0);
+    const size_t HW = (size_t)W * H;
+    for (int c0 = xr_lo; c0 < xr_hi; c0 += 64) {
+        for (int yr0 = yr_lo; yr0 < yr_hi; yr0 += SR) {
+            __syncthreads(); // the previous pass is no longer read
+            for (int i = tid; i < (SR + NW - 1) * 64; i += nthreads) {
+                const int r = i >> 6, c = i & 63;
+                const int yl = yr0 + sy0 + r, xr = c0 + c;
+                T v = T(0);
+                if (yl >= 0 && yl < H && xr < xr_hi) v = left[(size_t)yl * W + (xr + sx)];
+                Ls[i] = v;
+            }
+            for (int i = tid; i < NR * SR * 64; i += nthreads) {
+                const int c = i & 63, r = (i >> 6) % SR, m = (i >> 6) / SR;
+                const int yr = yr0 + r, xr = c0 + c;
+                T v = T(0);
+                if (m < nr && yr < yr_hi && xr < xr_hi) v = right[(size_t)(m0 + m) * HW + (size_t)yr * W + xr];
+                Rs[i] = v;
+            }
+            __syncthreads();
+            const T *lp = Ls + w * 64 + lane;
+            const T *rp = Rs + lane;
+#pragma unroll 4
+            for (int r = 0; r < SR; ++r) {
+                const T l = lp[r * 64];
+#pragma unroll
+                for (int m = 0; m < NR; ++m) sum[m] += l * rp[(m * SR + r) * 64];
+            }
+        }
+    }
+    if (oy >= Sy) return;
+#pragma unroll
+    for (int m = 0; m < NR; ++m) {
+        const T total = wave_sum_to_lane63(sum[m]);
+        if (lane == 63 && m < nr) {
+            T *p = out + (size_t)(m0 + m) * Sx * Sy + (size_t)oy * Sx + ox;
+            if (gridDim.z > 1)
+                atomic_add_simple(p, total);
+            else
+                *p = total;
+        }
+    }
+}
+
+template <typename T, int NR>
+static void launch_wpo_lds(const T *left, const T *right, T *out, int W, int H, int n_right, int SR, dim3 grid, dim3 block,
+                           size_t lds, hipStream_t stream) {
+    warp_per_overlap_lds_kernel<T, NR><<<grid, block, lds, stream>>>(left, right, out, W, H, n_right, SR);
+}
+
+// One left matrix against n_right right matrices (reference run_ccn_warp_per_shift_shared_mem,
+// naive_warp_per_shift_shared_mem.cu:610-700).
+template <typename T>
+int run_warp_per_overlap_lds(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_right,
+                             const xcorr_params &p, hipStream_t stream) {
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if (n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "warp_per_overlap_lds: no right matrices");
+    // reference limits: naive_warp_per_shift_shared_mem.cu:681-693
+    if (p.shifts_per_thread_block > 32)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "Too many shifts per block: %u (max 32)", p.shifts_per_thread_block);
+    unsigned nr = p.right_matrices_per_block ? p.right_matrices_per_block : 1;
+    if (nr > 8) return fail(XCORR_ERR_INVALID_ARGUMENT, "Invalid number of right matrices per block: %u [1-8]", nr);
+    unsigned nw = p.shifts_per_thread_block ? p.shifts_per_thread_block : 16;
+    if (nw > 16) nw = 16; // a block holds at most 16 wavefronts of 64 lanes
+    unsigned sr = p.shared_mem_rows ? p.shared_mem_rows : nw;
+    if (sr < nw) return fail(XCORR_ERR_INVALID_ARGUMENT, "Invalid number of shared memory rows [%u], must be greater than shifts per block [%u]", sr, nw);
+    // columns are staged 64 at a time (one per lane), whatever shared_mem_row_size asks for; the
+    // rows per pass are cut down until the bands fit 64 KB of LDS (the kernel itself works with
+    // any number of rows per pass; the rule above is the reference's)
+    auto lds_bytes = [&](unsigned r) { return ((size_t)(nr + 1) * r + nw - 1) * 64 * sizeof(T); };
+    while (sr > 1 && lds_bytes(sr) > 64 * 1024) sr /= 2;
+    const size_t lds = lds_bytes(sr);
+    if (lds > 64 * 1024) return fail(XCORR_ERR_UNSUPPORTED, "warp_per_overlap_lds: %zu bytes of LDS needed (max 65536)", lds);
+    const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
+    const unsigned groups = (n_right + nr - 1) / nr;
+    const unsigned column_groups = p.column_group_per_block ? (cols + 63) / 64 : 1;
+    dim3 block(64, nw), grid(Sx * groups, (Sy + nw - 1) / nw, column_groups);
+    const int W = (int)cols, H = (int)rows;
+    switch (nr) {
+    case 1: launch_wpo_lds<T, 1>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 2: launch_wpo_lds<T, 2>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 3: launch_wpo_lds<T, 3>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 4: launch_wpo_lds<T, 4>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 5: launch_wpo_lds<T, 5>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 6: launch_wpo_lds<T, 6>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    case 7: launch_wpo_lds<T, 7>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    default: launch_wpo_lds<T, 8>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
+    }
+    XCORR_HIP(hipGetLastError());
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "warp_per_overlap_lds/%s_r%u", sizeof(T) == 4 ? "f32" : "f64", nr);
+    rec.block[0] = block.x, rec.block[1] = block.y, rec.block[2] = 1;
+    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = grid.z;
+    rec.shared_mem_bytes = (unsigned)lds;
+    rec.y_shifts_per_thread = rec.x_shifts_per_thread = 1;
+    rec.left_matrices_per_thread = 1;
+    rec.right_matrices_per_thread = nr;
+    rec.rows_per_worker = sr;
+    rec.distribution_type = XCORR_DIST_NONE;
+    rec.uses_atomics = column_groups > 1;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+// ------------------------------------------------------------------ block-per-overlap
+// One block per shift: wavefront w takes the overlap rows w, w + NW, ..., lanes stride the
+// columns; wavefront sums meet in LDS and wavefront 0 adds them in order.
+template <typename T>
+__global__ __launch_bounds__(1024) void block_per_overlap_kernel(const T *__restrict__ left, const T *__restrict__ right,
+                                                                  T *__restrict__ out, int W, int H) {
+    __shared__ T partial[16];
+    const int Sx = 2 * W - 1;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int ox = blockIdx.x, oy = blockIdx.y;
+    const int sx = ox - (W - 1), sy = oy - (H - 1);
+    const int xr_lo = sx < 0 ? -sx : 0, xr_hi = W - sx < W ? W - sx : W;
+    const int yr_lo = sy < 0 ? -sy : 0, yr_hi = H - sy < H ? H - sy : H;
+    T part_sum[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) part_sum[r] = T(0);
+    for (int xr = xr_lo + lane; xr < xr_hi; xr += 64) {
+        int yr = yr_lo + w;
+        for (; yr + 3 * nw < yr_hi; yr += 4 * nw) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                part_sum[r] += left[(size_t)(yr + r * nw + sy) * W + (xr + sx)] * right[(size_t)(yr + r * nw) * W + xr];
+        }
+        for (; yr < yr_hi; yr += nw) part_sum[0] += left[(size_t)(yr + sy) * W + (xr + sx)] * right[(size_t)yr * W + xr];
+    }
+    T sum = wave_sum_to_lane63((part_sum[0] + part_sum[1]) + (part_sum[2] + part_sum[3]));
+    if (lane == 63) partial[w] = sum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        T total = partial[0];
+        for (int i = 1; i < nw; ++i) total += partial[i];
+        out[(size_t)oy * Sx + ox] = total;
+    }
+}
+
+// reference run_ccn_block_per_shift, naive_block_per_shift.cu:127-160
+template <typename T>
+int run_block_per_overlap(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params &p,
+                          hipStream_t stream) {
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    const unsigned asked = p.block_size ? p.block_size : 128; // reference default one_to_one.hpp:649
+    if (asked > 1024) return fail(XCORR_ERR_INVALID_ARGUMENT, "Thread block too large: %u (max 1024)", asked);
+    unsigned threads = asked / 64 * 64; // whole wavefronts
+    if (threads == 0) threads = 64;
+    dim3 block(threads), grid(2 * cols - 1, 2 * rows - 1);
+    block_per_overlap_kernel<T><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows);
+    XCORR_HIP(hipGetLastError());
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "block_per_overlap/%s", sizeof(T) == 4 ? "f32" : "f64");
+    rec.block[0] = block.x, rec.block[1] = rec.block[2] = 1;
+    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = 1;
+    rec.shared_mem_bytes = 16 * sizeof(T);
+    rec.y_shifts_per_thread = rec.x_shifts_per_thread = 1;
+    rec.left_matrices_per_thread = rec.right_matrices_per_thread = 1;
+    rec.rows_per_worker = rows;
+    rec.distribution_type = XCORR_DIST_NONE;
     have_last_launch() = true;
     return XCORR_OK;
 }

@@ -344,6 +344,24 @@ int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *
     return run_warp_per_overlap<double>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
 }
 
+int xcorr_warp_per_overlap_lds_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                   unsigned n_right, const xcorr_params *p, void *stream) {
+    return run_warp_per_overlap_lds<float>(left, right, out, cols, rows, n_right, params_or_default(p), as_stream(stream));
+}
+int xcorr_warp_per_overlap_lds_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                   unsigned n_right, const xcorr_params *p, void *stream) {
+    return run_warp_per_overlap_lds<double>(left, right, out, cols, rows, n_right, params_or_default(p), as_stream(stream));
+}
+
+int xcorr_block_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                const xcorr_params *p, void *stream) {
+    return run_block_per_overlap<float>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+}
+int xcorr_block_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                const xcorr_params *p, void *stream) {
+    return run_block_per_overlap<double>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+}
+
 #define XCORR_PAIR_ENTRY(NAME, IMPL)                                                                              \
     int NAME##_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,               \
                    const xcorr_params *p, void *stream) {                                                         \

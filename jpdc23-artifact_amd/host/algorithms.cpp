@@ -21,11 +21,11 @@ A streams() { return {"num_cuda_streams", U, 8, nullptr}; }
 
 std::vector<A> shared_mem_args(long long shifts_default, bool with_right_mats, bool with_streams) {
     std::vector<A> v{{"shifts_per_thread_block", U, shifts_default, &P::shifts_per_thread_block},
-                     {"shared_mem_row_size", U, 32, nullptr},
-                     {"shared_mem_rows", U, -1, nullptr}, // default: shifts_per_thread_block
-                     {"strided_load", B, 1, nullptr},
-                     {"column_group_per_block", B, 0, nullptr}};
-    if (with_right_mats) v.push_back({"right_matrices_per_block", U, 8, &P::right_matrices_per_thread});
+                     {"shared_mem_row_size", U, 32, &P::shared_mem_row_size},
+                     {"shared_mem_rows", U, -1, &P::shared_mem_rows}, // default: shifts_per_thread_block
+                     {"strided_load", B, 1, &P::strided_load},
+                     {"column_group_per_block", B, 0, &P::column_group_per_block}};
+    if (with_right_mats) v.push_back({"right_matrices_per_block", U, 8, &P::right_matrices_per_block});
     if (with_streams) v.push_back(streams());
     return v;
 }
@@ -140,20 +140,20 @@ std::vector<algorithm_def> build_defs() {
     }
     // shared-memory warp-per-shift (one_to_one.hpp:561, one_to_many.hpp:411, n_to_mn.hpp:575,
     // n_to_m.hpp:529): the LDS-staged engine families stand in for it
-    add("nai_warp_per_shift_shared_mem_one_to_one", Mode::one_to_one, Family::warp_per_overlap, shared_mem_args(32, false, false))
+    add("nai_warp_per_shift_shared_mem_one_to_one", Mode::one_to_one, Family::warp_per_overlap_lds, shared_mem_args(32, false, false))
         .shared_mem_rows_rule = true;
-    add("nai_warp_per_shift_shared_mem_one_to_many", Mode::one_to_many, Family::multimat_right_grouped, shared_mem_args(16, true, false))
+    add("nai_warp_per_shift_shared_mem_one_to_many", Mode::one_to_many, Family::warp_per_overlap_lds, shared_mem_args(16, true, false))
         .shared_mem_rows_rule = true;
     {
-        auto &a = add("nai_warp_per_shift_shared_mem_n_to_mn", Mode::n_to_mn, Family::multimat_right_grouped, shared_mem_args(16, true, true));
+        auto &a = add("nai_warp_per_shift_shared_mem_n_to_mn", Mode::n_to_mn, Family::warp_per_overlap_lds, shared_mem_args(16, true, true));
         a.shared_mem_rows_rule = a.per_left_streams = a.deinterleave = true;
     }
     {
-        auto &a = add("nai_warp_per_shift_shared_mem_n_to_m", Mode::n_to_m, Family::multimat_right_grouped, shared_mem_args(16, true, true));
+        auto &a = add("nai_warp_per_shift_shared_mem_n_to_m", Mode::n_to_m, Family::warp_per_overlap_lds, shared_mem_args(16, true, true));
         a.shared_mem_rows_rule = a.per_left_streams = true;
     }
-    // block-per-shift (one_to_one.hpp:644): one wavefront per shift stands in for it
-    add("nai_block_per_shift_one_to_one", Mode::one_to_one, Family::warp_per_overlap, {{"block_size", U, 128, nullptr}}).block_size_limit = 1024;
+    // block-per-shift (one_to_one.hpp:644)
+    add("nai_block_per_shift_one_to_one", Mode::one_to_one, Family::block_per_overlap, {{"block_size", U, 128, &P::block_size}});
     return d;
 }
 
@@ -163,6 +163,8 @@ template <>
 struct entry<float> {
     static constexpr auto overlap_wise = xcorr_overlap_wise_f32;
     static constexpr auto warp_per_overlap = xcorr_warp_per_overlap_f32;
+    static constexpr auto warp_per_overlap_lds = xcorr_warp_per_overlap_lds_f32;
+    static constexpr auto block_per_overlap = xcorr_block_per_overlap_f32;
     static constexpr auto shuffle = xcorr_shuffle_f32;
     static constexpr auto split_row = xcorr_split_row_f32;
     static constexpr auto grouped_overlap = xcorr_grouped_overlap_f32;
@@ -175,6 +177,8 @@ template <>
 struct entry<double> {
     static constexpr auto overlap_wise = xcorr_overlap_wise_f64;
     static constexpr auto warp_per_overlap = xcorr_warp_per_overlap_f64;
+    static constexpr auto warp_per_overlap_lds = xcorr_warp_per_overlap_lds_f64;
+    static constexpr auto block_per_overlap = xcorr_block_per_overlap_f64;
     static constexpr auto shuffle = xcorr_shuffle_f64;
     static constexpr auto split_row = xcorr_split_row_f64;
     static constexpr auto grouped_overlap = xcorr_grouped_overlap_f64;
@@ -263,18 +267,8 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
                                  "], must be greater than shifts per block [" + std::to_string(shifts_per_thread_block) + "]",
                              "shared_mem_rows");
     }
-    if (def.shared_mem_rows_rule) {
-        // the staged engine has its own band geometry; the request is honoured as far as its limits go
-        if (params_.right_matrices_per_thread > 4) params_.right_matrices_per_thread = 4;
-        if (def.family == Family::warp_per_overlap) params_.warp_per_overlap_variant = XCORR_WPO_SIMPLE_INDEXING;
-        if (def.family != Family::warp_per_overlap) params_.shifts_per_thread_block = 0;
-    }
-    if (def.block_size_limit) {
-        unsigned block_size = args.value("block_size", 128u);
-        if (block_size > def.block_size_limit) // naive_block_per_shift.cu:136-140
-            throw std::runtime_error("Too many threads per block: " + std::to_string(block_size) + " (max " + std::to_string(def.block_size_limit) + ")");
-        params_.shifts_per_thread_block = std::max(1u, block_size / 64);
-    }
+    // (the shifts-per-block and block-size limits are the launchers': they fail in the first launch, exit code 3)
+    zero_output_ = def.zero_output || (def.family == Family::warp_per_overlap_lds && params_.column_group_per_block);
     if (def.fixed_one_right_per_thread) params_.right_matrices_per_thread = 1;
     if (def.per_left_streams && num_streams_ == 0) num_streams_ = 1;
     // the unpublished "multirow_right" kernels allow up to 8 rows, the combined engine tiles 4
@@ -328,6 +322,8 @@ void gpu_algorithm<T>::launch(const T *left, const T *right, T *out, dsize_t n_l
     switch (def_.family) {
     case Family::overlap_wise: xcheck(E::overlap_wise(left, right, out, cols, rows, n_left, n_right, stream)); break;
     case Family::warp_per_overlap: xcheck(E::warp_per_overlap(left, right, out, cols, rows, &params_, stream)); break;
+    case Family::warp_per_overlap_lds: xcheck(E::warp_per_overlap_lds(left, right, out, cols, rows, n_right, &params_, stream)); break;
+    case Family::block_per_overlap: xcheck(E::block_per_overlap(left, right, out, cols, rows, &params_, stream)); break;
     case Family::shuffle: xcheck(E::shuffle(left, right, out, cols, rows, &params_, stream)); break;
     case Family::split_row: xcheck(E::split_row(left, right, out, cols, rows, &params_, stream)); break;
     case Family::grouped_overlap: xcheck(E::grouped_overlap(left, right, out, cols, rows, &params_, stream)); break;
@@ -346,9 +342,9 @@ template <typename T>
 void gpu_algorithm<T>::launch_all() {
     const dsize_t n = refs_.num_matrices(), total_right = targets_.num_matrices();
     const std::size_t in_area = refs_.matrix_size().area(), out_area = results_.matrix_size().area();
-    if (def_.zero_output) xcheck(xcorr_memset_async(d_results_, 0, results_.size() * sizeof(T), nullptr));
+    if (zero_output_) xcheck(xcorr_memset_async(d_results_, 0, results_.size() * sizeof(T), nullptr));
     if (def_.per_left_streams) {
-        if (def_.zero_output) xcheck(xcorr_device_sync()); // the clear runs on the default stream
+        if (zero_output_) xcheck(xcorr_device_sync()); // the clear runs on the default stream
         // one launch per left matrix, left r on stream r mod k (n_to_mn.hpp:553-571, n_to_m.hpp:198-212)
         const bool all_pairs = def_.mode == Mode::n_to_m;
         const dsize_t per_left = all_pairs ? total_right : total_right / n;

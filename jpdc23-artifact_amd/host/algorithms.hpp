@@ -182,6 +182,8 @@ private:
 enum class Family {
     overlap_wise,
     warp_per_overlap,
+    warp_per_overlap_lds,
+    block_per_overlap,
     shuffle,
     split_row,
     grouped_overlap,
@@ -214,7 +216,6 @@ struct algorithm_def {
     unsigned wpo_variant = 0;
     bool fixed_one_right_per_thread = false; // *_one_to_one flavours of the multi-matrix kernels
     bool shared_mem_rows_rule = false;       // argument_error rule of the shared-memory variants
-    unsigned block_size_limit = 0;           // nai_block_per_shift: block_size <= 1024
 };
 
 const std::vector<algorithm_def> &gpu_algorithm_defs();
@@ -248,6 +249,7 @@ protected:
 private:
     algorithm_def def_;
     xcorr_params params_{};
+    bool zero_output_ = false; // clear the output inside the measured block (split-row contract, column groups)
     properties props_;
     unsigned num_streams_ = 0;
     host_array refs_, targets_, results_;

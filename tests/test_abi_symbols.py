@@ -18,7 +18,7 @@ def declared_symbols():
 
 def test_header_declares_the_expected_surface():
     names = declared_symbols()
-    for family in ["overlap_wise", "warp_per_overlap", "shuffle", "split_row", "grouped_overlap", "multimat_right",
+    for family in ["overlap_wise", "warp_per_overlap", "warp_per_overlap_lds", "block_per_overlap", "shuffle", "split_row", "grouped_overlap", "multimat_right",
                    "multimat_right_grouped", "multimat_both", "multimat_both_grouped"]:
         assert f"xcorr_{family}_f32" in names and f"xcorr_{family}_f64" in names
     assert len(names) >= 40
@@ -60,6 +60,18 @@ def test_argument_errors_without_a_device():
     assert b"Unknown distribution" in lib.xcorr_last_error()
     p = xc.make_params(right_matrices_per_thread=5)
     assert lib.xcorr_multimat_both_grouped_f32(dummy, dummy, dummy, 8, 8, 2, 2, ctypes.byref(p), None) == 1
+    p = xc.make_params(shifts_per_thread_block=33)
+    assert lib.xcorr_warp_per_overlap_lds_f32(dummy, dummy, dummy, 8, 8, 1, ctypes.byref(p), None) == 1
+    assert b"Too many shifts per block: 33 (max 32)" in lib.xcorr_last_error()
+    p = xc.make_params(right_matrices_per_block=9)
+    assert lib.xcorr_warp_per_overlap_lds_f32(dummy, dummy, dummy, 8, 8, 1, ctypes.byref(p), None) == 1
+    assert b"Invalid number of right matrices per block: 9 [1-8]" in lib.xcorr_last_error()
+    p = xc.make_params(shifts_per_thread_block=8, shared_mem_rows=4)
+    assert lib.xcorr_warp_per_overlap_lds_f64(dummy, dummy, dummy, 8, 8, 1, ctypes.byref(p), None) == 1
+    assert b"Invalid number of shared memory rows [4]" in lib.xcorr_last_error()
+    p = xc.make_params(block_size=2048)
+    assert lib.xcorr_block_per_overlap_f32(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None) == 1
+    assert b"Thread block too large: 2048 (max 1024)" in lib.xcorr_last_error()
     rec = xc.LaunchRecord()
     assert lib.xcorr_last_launch(ctypes.byref(rec)) == 1
     assert b"No kernel launch" in lib.xcorr_last_error()

@@ -69,6 +69,14 @@ ONE_TO_ONE_CASES = [
     ("multimat_right_grouped", {}),
     ("multimat_both", {}),
     ("multimat_both_grouped", {}),
+    ("warp_per_overlap_lds", {}),
+    ("warp_per_overlap_lds", dict(shifts_per_thread_block=32, shared_mem_rows=32)),
+    ("warp_per_overlap_lds", dict(shifts_per_thread_block=3, shared_mem_rows=7)),
+    ("warp_per_overlap_lds", dict(shifts_per_thread_block=8, column_group_per_block=1)),
+    ("block_per_overlap", {}),
+    ("block_per_overlap", dict(block_size=64)),
+    ("block_per_overlap", dict(block_size=1024)),
+    ("block_per_overlap", dict(block_size=200)),
 ]
 
 
@@ -101,6 +109,10 @@ ONE_TO_MANY_CASES = [
     ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=2, right_matrices_per_thread=2, rows_per_thread=16)),
     ("multimat_both", dict(left_matrices_per_thread=1, right_matrices_per_thread=4)),
     ("multimat_both_grouped", {}),
+    ("warp_per_overlap_lds", dict(right_matrices_per_block=1)),
+    ("warp_per_overlap_lds", dict(right_matrices_per_block=8, shifts_per_thread_block=16)),
+    ("warp_per_overlap_lds", dict(right_matrices_per_block=3, shifts_per_thread_block=5, shared_mem_rows=9)),
+    ("warp_per_overlap_lds", dict(right_matrices_per_block=4, shifts_per_thread_block=8, column_group_per_block=1)),
 ]
 
 
