@@ -396,11 +396,10 @@ void gpu_algorithm<T>::free_impl() {
 
 template <typename T>
 void gpu_algorithm<T>::store_results_impl(const std::filesystem::path &out) const {
-    std::ofstream file{out};
     if (def_.deinterleave) // back to the file order of the inputs (n_to_mn.hpp:515-519)
-        results_.store_interleaved_to_csv(file, targets_.num_matrices() / refs_.num_matrices());
+        results_.store_interleaved(out, targets_.num_matrices() / refs_.num_matrices());
     else
-        results_.store_to_csv(file);
+        results_.store(out);
 }
 
 template <typename T>

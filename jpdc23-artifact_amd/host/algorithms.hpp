@@ -168,10 +168,7 @@ protected:
         default: cpu_cross_corr_n_to_m(refs_, targets_, results_); break;
         }
     }
-    void store_results_impl(const std::filesystem::path &out) const override {
-        std::ofstream file{out};
-        results_.store_to_csv(file);
-    }
+    void store_results_impl(const std::filesystem::path &out) const override { results_.store(out); }
 
 private:
     Mode mode_;

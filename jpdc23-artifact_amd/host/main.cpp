@@ -115,6 +115,7 @@ void print_help(std::ostream &out, const std::string &name) {
     out << "\t" << name << " [global options] run [run options] <alg> <ref_path> <target_path>\n";
     out << "\t" << name << " [global options] validate [validate options] <validate_data_path> <template_data_path>\n";
     out << "\t" << name << " [global options] input [input options] <alg_type> <rows> <columns> <left_matrices> <right_matrices>\n";
+    out << "\t" << name << " [global options] convert <in_path> <out_path>   (text <-> binary matrix file; \".bin\" selects binary)\n";
     out << "Global options:\n  -h [ --help ]                         display this help and exit\n";
     out << "Validate options:\n"
            "  -n [ --normalize ]                    Normalize the data to be validated as they are denormalized fft output\n"
@@ -399,6 +400,15 @@ int cmd_validate(const std::vector<std::string> &args) {
     return 0;
 }
 
+// Not in the reference: rewrites a matrix file in the other format (the extension of the output
+// path decides), so large inputs are parsed from text only once.
+int cmd_convert(const std::vector<std::string> &args) {
+    parsed_options o = parse_options(args, no_option_defs);
+    if (o.positional.size() != 2) throw cli_error("convert expects <in_path> <out_path>");
+    load_matrix_array_from_csv<double>(o.positional[0]).store(o.positional[1]);
+    return 0;
+}
+
 // main.cpp:328-359
 int cmd_input(const std::vector<std::string> &args, const std::string &prog) {
     parsed_options o = parse_options(args, no_option_defs);
@@ -461,6 +471,8 @@ int main(int argc, char **argv) {
             return 0;
         } else if (cmd == "input") {
             return cmd_input(sub, prog);
+        } else if (cmd == "convert") {
+            return cmd_convert(sub);
         }
         std::cerr << "Unknown command " << cmd << "\n";
         print_help(std::cerr, prog);

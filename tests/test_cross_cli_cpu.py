@@ -175,3 +175,86 @@ def test_exit_codes(tmp_path):
     (tmp_path / "c.json").write_text("{ not json")
     rc, _, err = run_cross("run", "--args_path", tmp_path / "c.json", "nai_shuffle_one_to_one", lp, lp)
     assert rc == 2 and "JSON arguments" in err
+
+
+def _matrix_io():
+    from conftest import load_package
+    import importlib.util
+    xc = load_package()
+    spec = importlib.util.spec_from_file_location("xcorr_matrix_io", os.path.join(xc.PKG_DIR, "matrix_io.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def test_binary_matrix_files_keep_every_bit(tmp_path, oracle):
+    """Binary inputs and a '.bin' output path: the result file holds the computed floats
+    themselves (the text format rounds to six decimals), so the comparison with the oracle is
+    exact for real-valued data too. Mode n_to_mn exercises the interleaved reader / writer."""
+    mio = _matrix_io()
+    rng = np.random.default_rng(42)
+    left = rng.standard_normal((2, 5, 7)).astype(np.float32)
+    right = rng.standard_normal((6, 5, 7)).astype(np.float32)
+    lp, rp = mio.write_binary(tmp_path / "l.bin", left), mio.write_binary(tmp_path / "r.bin", right)
+    out = tmp_path / "o.bin"
+    rc, _, err = run_cross("run", "-o", out, "cpu_n_to_mn", lp, rp)
+    assert rc == 0, err
+    got = mio.read_binary(out)
+    assert got.dtype == np.float32
+    exp = oracle.n_to_mn(left, right)
+    assert np.array_equal(got, exp)
+    # a double-precision file read by a single-precision run is converted on load
+    lp64 = mio.write_binary(tmp_path / "l64.bin", left.astype(np.float64))
+    rc, _, err = run_cross("run", "-o", tmp_path / "o2.bin", "cpu_n_to_mn", lp64, rp)
+    assert rc == 0, err
+    assert np.array_equal(mio.read_binary(tmp_path / "o2.bin"), exp)
+    # and --data_type double writes 8-byte elements
+    rc, _, err = run_cross("run", "-d", "double", "-o", tmp_path / "o3.bin", "cpu_n_to_mn", lp, rp)
+    assert rc == 0, err
+    got64 = mio.read_binary(tmp_path / "o3.bin")
+    assert got64.dtype == np.float64
+    assert np.array_equal(got64, oracle.n_to_mn(left.astype(np.float64), right.astype(np.float64)))
+
+
+def test_convert_subcommand_and_bad_binary_files(tmp_path):
+    mio = _matrix_io()
+    a = np.arange(2 * 3 * 4, dtype=np.float64).reshape(2, 3, 4) / 8
+    text = write_matrices(tmp_path / "a.csv", a)
+    rc, _, err = run_cross("convert", text, tmp_path / "a.bin")
+    assert rc == 0, err
+    assert np.array_equal(mio.read_binary(tmp_path / "a.bin"), a)
+    rc, _, err = run_cross("convert", tmp_path / "a.bin", tmp_path / "b.csv")
+    assert rc == 0, err
+    assert np.array_equal(read_matrices(tmp_path / "b.csv"), a)
+    assert open(tmp_path / "b.csv").readline() == "# 3,4,2\n"
+    assert open(tmp_path / "b.csv").readlines()[1] == "0.000000,0.125000,0.250000,0.375000\n"
+    # truncated data and wrong version are reported, exit code 2 like any malformed input
+    blob = open(tmp_path / "a.bin", "rb").read()
+    open(tmp_path / "short.bin", "wb").write(blob[:-8])
+    rc, _, err = run_cross("convert", tmp_path / "short.bin", tmp_path / "c.csv")
+    assert rc == 2 and "too short" in err
+    open(tmp_path / "ver.bin", "wb").write(blob[:8] + (7).to_bytes(4, "little") + blob[12:])
+    rc, _, err = run_cross("convert", tmp_path / "ver.bin", tmp_path / "c.csv")
+    assert rc == 2 and "Unsupported" in err
+    rc, _, err = run_cross("convert", text)
+    assert rc == 1
+
+
+def test_csv_lines_with_and_without_quoting_parse_alike(tmp_path):
+    """Plain lines are parsed in place, lines with quotes or escapes go through the field
+    splitter (boost escaped_list_separator rules of the reference): same values either way;
+    std::stof semantics (leading blanks, trailing characters, exponents, hex, inf) in both."""
+    plain = tmp_path / "p.csv"
+    quoted = tmp_path / "q.csv"
+    open(plain, "w").write("# 2,4,1\n 1.5,-2e-3,0x10,7abc\ninf,-0.0,+3,.5e1\n")
+    open(quoted, "w").write('# 2,4,1\n" 1.5",-2e-3,"0x10",7abc\ninf,\\-0.0,+3,".5e1"\n')
+    for src in (plain, quoted):
+        rc, _, err = run_cross("convert", src, tmp_path / "o.bin")
+        assert rc == 0, err
+        got = _matrix_io().read_binary(tmp_path / "o.bin")[0]
+        assert np.array_equal(got, np.array([[1.5, -2e-3, 16.0, 7.0], [np.inf, -0.0, 3.0, 5.0]]))
+        assert np.signbit(got[1, 1])
+    for body, what in [("1,2,3\n", "too short"), ("1,2,3,4,5\n", "too long"), ("1,,3,4\n", "sto"), ("1,x,3,4\n", "sto")]:
+        open(plain, "w").write("# 1,4,1\n" + body)
+        rc, _, err = run_cross("convert", plain, tmp_path / "o.bin")
+        assert rc == 2 and what in err, (body, err)
