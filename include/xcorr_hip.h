@@ -56,10 +56,13 @@ extern "C" {
 /*
  * Tuning integers, named after the reference's per-algorithm JSON keys
  * (one_to_one.hpp:739-741, n_to_m.hpp:321-325, n_to_m.hpp:475-479, ...). The
- * reference counts 32-lane warps; this library runs 64-lane wavefronts and maps
- * a request onto the nearest gfx950 specialisation, see xcorr_last_launch().
- * Upper limits are the reference's release limits (CMakeLists.txt:16-46); larger
- * values are rejected as there.
+ * reference counts 32-lane warps and instantiates one kernel per value; this
+ * library runs a short list of gfx950 tiles on 64-lane wavefronts and picks the one
+ * its cost model rates best for the sizes at hand. The integers are checked against
+ * the reference's release limits (CMakeLists.txt:16-46; larger values are rejected
+ * as there) and otherwise only break ties between equally rated tiles; the tile
+ * actually used is reported by xcorr_last_launch(). The geometry fields further down
+ * select a tile exactly.
  */
 typedef struct xcorr_params {
     unsigned warps_per_thread_block;         /* <= 32 */

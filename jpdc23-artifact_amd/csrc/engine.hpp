@@ -94,7 +94,7 @@ struct EngineCfg {
     static constexpr int LDS_BUFFERS = DB ? 2 : 1;
     static constexpr int LDS_BYTES = (LDS_ELEMS * LDS_BUFFERS > RED_ELEMS ? LDS_ELEMS * LDS_BUFFERS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
-    static_assert(WZ == 1 || (WX == 1 && WY == 1 && A % WZ == 0), "row-splitting wavefronts share one wavefront tile");
+    static_assert(WZ == 1 || (WX == 1 && WY == 1 && (A % WZ == 0 || A < WZ)), "row-splitting wavefronts share one wavefront tile");
     static_assert((KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -582,11 +582,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         // all WZ versions of its own row (in wavefront order, so the result is deterministic).
         T *red = reinterpret_cast<T *>(smem_raw);
         constexpr int RR = C::RED_ROW;
+        // tile rows summed per pass: one per wavefront, or a single one (by wavefront 0) when
+        // the tile has fewer rows than the block has wavefronts
+        constexpr int OWN = A % C::WZ == 0 ? C::WZ : 1;
 #pragma unroll
-        for (int q = 0; q < A / C::WZ; ++q) {
+        for (int q = 0; q < A / OWN; ++q) {
             __syncthreads(); // bands, or the previous pass, are no longer read
 #pragma unroll
-            for (int o = 0; o < C::WZ; ++o) {
+            for (int o = 0; o < OWN; ++o) {
                 T *dst = red + ((size_t)(o * C::WZ + group) * 64 + lane) * RR;
 #pragma unroll
                 for (int i = 0; i < NV; ++i)
@@ -596,11 +599,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                         for (int b = 0; b < B; b += VK) {
                             vec piece;
 #pragma unroll
-                            for (int e = 0; e < VK; ++e) piece[e] = acc[i][n][q * C::WZ + o][b + e];
+                            for (int e = 0; e < VK; ++e) piece[e] = acc[i][n][q * OWN + o][b + e];
                             *reinterpret_cast<vec *>(dst + (i * NU + n) * B + b) = piece;
                         }
             }
             __syncthreads();
+            if (group >= OWN) continue;
             T sum[NV][NU][B];
 #pragma unroll
             for (int src = 0; src < C::WZ; ++src) {
@@ -616,7 +620,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                             for (int e = 0; e < VK; ++e) sum[i][n][b + e] = src == 0 ? piece[e] : sum[i][n][b + e] + piece[e];
                         }
             }
-            const int oy = oy0 + q * C::WZ + group;
+            const int oy = oy0 + q * OWN + group;
             if (oy < 0 || oy >= Sy) continue;
 #pragma unroll
             for (int i = 0; i < NV; ++i) {

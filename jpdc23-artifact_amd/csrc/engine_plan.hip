@@ -38,7 +38,7 @@ static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)
 //     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower (fp64: 8x8 5 % slower);
 //   * lanes laid over matrices stage one band per matrix, and a right band carries a halo of
 //     TYW-1 rows: +2.8 % per extra right matrix, +2 % per extra left matrix.
-// Hints scale the cost so the nearest specialisation wins without excluding the others.
+// Hints scale the cost a little so that the nearest of equally good specialisations wins.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
     double waste_y = std::sqrt((double)(rq.H + s.TYW()) * (rq.H + s.TYB())) / rq.H;
@@ -60,10 +60,12 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
     if (s.WX * s.WY * s.WZ < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
     if (s.A > 1 && s.WZ == 1) cost *= 1.1; // shift-tiled blocks wait at the barriers of partial stages
-    if (rq.y_shifts > 1) cost *= 1.0 + 3.0 * log2_ratio(s.A, rq.y_shifts);
-    if (rq.left_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NV, rq.left_mats);
-    if (rq.right_mats) cost *= 1.0 + 3.0 * log2_ratio(s.NU, rq.right_mats);
-    if (rq.waves) cost *= 1.0 + 0.05 * log2_ratio(s.WX * s.WY * s.WZ, rq.waves);
+    // the reference's tuning integers were found for its own kernels on other hardware: they only
+    // break ties here (2 % per doubling away from the request)
+    if (rq.y_shifts > 1) cost *= 1.0 + 0.02 * log2_ratio(s.A, rq.y_shifts);
+    if (rq.left_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NV * s.LV, rq.left_mats);
+    if (rq.right_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NU * s.LU, rq.right_mats);
+    if (rq.waves) cost *= 1.0 + 0.01 * log2_ratio(s.WX * s.WY * s.WZ, rq.waves);
     return cost;
 }
 

@@ -98,7 +98,9 @@ std::vector<algorithm_def> build_defs() {
         std::vector<A> v = mrg;
         v.push_back(streams());
         auto &a = add("nai_shuffle_multirow_both_multimat_right_n_to_mn", Mode::n_to_mn, Family::multimat_right_grouped, v);
-        a.per_left_streams = a.deinterleave = true;
+        // one launch over all left matrices instead of the reference's launch per left matrix on
+        // num_cuda_streams streams (n_to_mn.hpp:553-571): the key is read and reported, not used
+        a.deinterleave = true;
     }
     // multi-matrix-both x grouped-overlap (n_to_m.hpp:470)
     add("nai_shuffle_multirow_both_multimat_both_n_to_m", Mode::n_to_m, Family::multimat_both_grouped,
@@ -122,7 +124,7 @@ std::vector<algorithm_def> build_defs() {
         std::vector<A> v = mrr;
         v.push_back(streams());
         auto &a = add("nai_shuffle_multirow_right_multimat_right_n_to_mn", Mode::n_to_mn, Family::multimat_right_grouped, v);
-        a.per_left_streams = a.deinterleave = true;
+        a.deinterleave = true; // one launch, as above
     }
     // warp-per-overlap (one_to_one.hpp:410, :519, :452)
     add("nai_warp_per_shift_one_to_one", Mode::one_to_one, Family::warp_per_overlap,
