@@ -17,9 +17,6 @@ namespace xcorr {
 using R_1x1 = EngineCfg<float, 1, 8, 4, 1, 1, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_1x4 = EngineCfg<float, 1, 8, 4, 1, 4, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_2x2 = EngineCfg<float, 1, 8, 4, 2, 2, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
-// several matrices per lane (the reference's left/right_matrices_per_thread), 2x2 wavefronts
-using G_48_n2 = EngineCfg<float, 4, 8, 4, 1, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
-using G_44_n22 = EngineCfg<float, 4, 4, 4, 2, 2, 8, 8, 1, 1, 2, 2, 20, 32, 4>;
 // grouped tiles: four wavefronts share one tile and its bands and take every fourth chunk of columns of
 // a stage (WZ = 4). Lanes over shifts only ...
 using Z_84 = EngineCfg<float, 8, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
@@ -33,13 +30,12 @@ using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 18, 16, 4, 4
 using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 18, 16, 4, 4>;
-using Z_84_u8a = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 4, 4>;
+using Z_84_u8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 4, 4>;
+
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),
     make_spec<R_1x4>("f32_a1b8_r4"),
     make_spec<R_2x2>("f32_a1b8_l2r2"),
-    make_spec<G_48_n2>("f32_a4b8_r2"),
-    make_spec<G_44_n22>("f32_a4b4_l2r2"),
     make_spec<Z_84>("f32_a8b4"),
     make_spec<Z_88>("f32_a8b8"),
     make_spec<Z_44>("f32_a4b4"),
@@ -50,7 +46,7 @@ static const EngineSpec specs[] = {
     make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4"),
     make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4"),
     make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8"),
-    make_spec<Z_84_u8a>("f32_a8b4_lr8"),
+    make_spec<Z_84_u8>("f32_a8b4_lr8"),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {
