@@ -17,12 +17,13 @@
 //     left / right matrices, so small matrices get narrow shift tiles (less work
 //     wasted on partial overlaps) without losing register-level reuse;
 //   * a block stages a band of RL left rows and the matching band of right rows in
-//     LDS, zero padded, so the inner loop has no bounds checks;
+//     LDS, zero padded, so the inner loop has no bounds checks; its wavefronts either own
+//     adjacent shift tiles (WX x WY) or share one tile and split its reduction (WZ);
 //   * per left row and K right columns a lane reads one B+K-1 wide left window and
 //     one new right row of K values; the A right rows it needs are kept in a
 //     register ring that rotates by one row per step (the y loop is unrolled so every
-//     ring index is static), and every LDS read is issued one step ahead of its use. That is NV*NU*A*B*K FMAs for
-//     NV*ceil((B+K-1)/v) + NU*ceil(K/v) 128-bit LDS reads (v = 16 / sizeof(T));
+//     ring index is static), and every LDS read is issued one step ahead of its use. That is
+//     NV*NU*A*B*K FMAs for NV*ceil((B+K-1)/v) + NU*ceil(K/v) 128-bit LDS reads (v = 16 / sizeof(T));
 //   * the reduction over left rows can be split into chunks (work items) whose
 //     partial sums are added with hardware float atomics, which is what fills 256
 //     CUs when a single large pair has only ~1000 wavefront tiles.
@@ -72,7 +73,7 @@ struct EngineCfg {
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
     static constexpr int NWAVES = WX * WY * WZ, NT = 64 * NWAVES;
-        static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
+    static constexpr int G = A + 1; // left rows per unrolled group = slots of the right-row ring
     static constexpr int VWIN = B + K - 1;
     static constexpr int VWIN_VECS = (VWIN + VK - 1) / VK;
     static constexpr int KVECS = K / VK;
@@ -94,7 +95,7 @@ struct EngineCfg {
     static constexpr int LDS_BUFFERS = DB ? 2 : 1;
     static constexpr int LDS_BYTES = (LDS_ELEMS * LDS_BUFFERS > RED_ELEMS ? LDS_ELEMS * LDS_BUFFERS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
-    static_assert(WZ == 1 || (WX == 1 && WY == 1 && (A % WZ == 0 || A < WZ)), "row-splitting wavefronts share one wavefront tile");
+    static_assert(WZ == 1 || (WX == 1 && WY == 1 && (A % WZ == 0 || A < WZ)), "wavefronts that split a reduction share one wavefront tile");
     static_assert((KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -215,9 +216,15 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
 // lds_base + 16 * i, without passing through registers; completion is counted by vmcnt. The
 // compiler does not know that this writes LDS: callers wait (dma_wait) and pass a barrier before
 // anything reads the destination.
+// (M0, which carries the LDS address, is a register the compiler reserves for uses of this
+// kind and never keeps a value in across statements; naming it as clobbered states the fact and
+// draws a warning about reserved registers, silenced here.)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 __device__ __forceinline__ void dma16(const void *gptr, unsigned lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_base) : "memory", "m0");
 }
+#pragma clang diagnostic pop
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // stage_bands with the copies done by dma16: pieces that lie fully inside the matrices are copied
@@ -369,7 +376,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     const int tid = (int)threadIdx.x;
-    const int group = C::WZ > 1 ? __builtin_amdgcn_readfirstlane(tid >> 6) : 0; // which share of the rows
+    const int group = C::WZ > 1 ? __builtin_amdgcn_readfirstlane(tid >> 6) : 0; // which share of the column chunks
     T *Vs = reinterpret_cast<T *>(smem_raw);
     T *Us = Vs + C::NVB * C::VBAND;
     const int W = g.W, H = g.H;
