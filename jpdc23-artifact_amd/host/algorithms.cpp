@@ -1,5 +1,6 @@
 // Algorithm registry (the reference's main.cpp:361-411) and the generic GPU algorithm.
 #include "algorithms.hpp"
+#include "fft_algorithms.hpp"
 
 #include <algorithm>
 
@@ -207,17 +208,10 @@ const std::vector<algorithm_def> &gpu_algorithm_defs() {
     return defs;
 }
 
-const std::vector<std::string> &unsupported_fft_names() {
-    // the cuFFT comparison path of the reference (main.cpp:403-409) is not part of this build
-    static const std::vector<std::string> names{"fft_orig_one_to_one",     "fft_reduced_transfer_one_to_one", "fft_orig_one_to_many",
-                                                "fft_reduced_transfer_one_to_many", "fft_orig_n_to_mn", "fft_reduced_transfer_n_to_mn",
-                                                "fft_better_n_to_m"};
-    return names;
-}
-
 std::vector<std::string> algorithm_names() {
     std::vector<std::string> names{"cpu_one_to_one", "cpu_one_to_many", "cpu_n_to_mn", "cpu_n_to_m"};
     for (auto &d : gpu_algorithm_defs()) names.push_back(d.name);
+    for (auto &d : fft_algorithm_defs()) names.push_back(d.name);
     std::sort(names.begin(), names.end());
     return names;
 }
@@ -436,6 +430,11 @@ std::unique_ptr<algorithm> make_algorithm(const std::string &name, const std::st
         if (d.name != name) continue;
         if (is_double) return std::make_unique<gpu_algorithm<double>>(d, args, bench, min_time);
         return std::make_unique<gpu_algorithm<float>>(d, args, bench, min_time);
+    }
+    for (auto &d : fft_algorithm_defs()) {
+        if (d.name != name) continue;
+        if (is_double) return std::make_unique<fft_algorithm<double>>(d, args, bench, min_time);
+        return std::make_unique<fft_algorithm<float>>(d, args, bench, min_time);
     }
     throw std::runtime_error("Invalid algorithm specified \"" + name + "\"");
 }

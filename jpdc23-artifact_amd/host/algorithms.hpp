@@ -82,8 +82,12 @@ public:
     virtual properties additional_properties() const { return {}; }
     virtual validation_results validate(const std::optional<std::filesystem::path> &valid_path) const = 0;
     virtual bool uses_device() const = 0;
+    virtual bool is_fft() const { return false; }
+    // --normalize: FFT algorithms store their results in the definition's layout (fft_alg.hpp:13-20)
+    void set_normalize(bool on) { normalize_ = on; }
 
 protected:
+    bool normalize_ = false;
     BenchmarkType bench_;
     stopwatch sw_;
     bool measure_common() const { return bench_ == BenchmarkType::CommonSteps; }
@@ -216,7 +220,6 @@ struct algorithm_def {
 };
 
 const std::vector<algorithm_def> &gpu_algorithm_defs();
-const std::vector<std::string> &unsupported_fft_names();
 
 template <typename T>
 struct device_entry_points;

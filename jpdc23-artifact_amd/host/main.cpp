@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "algorithms.hpp"
+#include "fft_algorithms.hpp"
 
 using namespace cross;
 namespace fs = std::filesystem;
@@ -279,6 +280,7 @@ int run_measurement(const run_args &ra) {
         alg_args = json_args::parse(args_file);
     }
     auto alg = make_algorithm(ra.alg_name, ra.data_type, alg_args, ra.benchmark_type, ra.min_time);
+    alg->set_normalize(ra.normalize); // main.cpp:176-187
 
     try {
         logger.log("Loading inputs");
@@ -360,11 +362,6 @@ int cmd_run(const std::vector<std::string> &args, const std::string &prog) {
     ra.append_measurements = o.has("append");
     ra.print_progress = !o.has("no_progress");
 
-    const auto &fft = unsupported_fft_names();
-    if (std::find(fft.begin(), fft.end(), ra.alg_name) != fft.end()) {
-        std::cerr << "Algorithm \"" << ra.alg_name << "\" belongs to the FFT comparison path, which this build does not contain" << std::endl;
-        return 1;
-    }
     if (!is_algorithm(ra.alg_name)) { // run_args.cpp:108-111
         std::cerr << "Unknown algorithm \"" << ra.alg_name << "\", expected one of " << join(algorithm_names()) << std::endl;
         print_help(std::cerr, prog);
@@ -388,13 +385,14 @@ int cmd_validate(const std::vector<std::string> &args) {
     parsed_options o = parse_options(args, validate_option_defs);
     if (o.positional.empty()) throw cli_error("the option '--template_data_path' is required but missing");
     if (o.positional.size() < 2) throw cli_error("the option '--validate_data_path' is required but missing");
-    if (o.has("normalize")) throw cli_error("--normalize applies to FFT results, which this build does not produce");
+    const bool normalize = o.has("normalize");
     const bool csv = o.has("csv"), print_header = o.has("print_header");
     simple_logger logger{!csv, true};
     auto valid = load_matrix_array_from_csv<double>(o.positional[0]);
     for (std::size_t i = 1; i < o.positional.size(); ++i) {
         logger.log("Validating " + o.positional[i]);
         auto target = load_matrix_array_from_csv<double>(o.positional[i]);
+        if (normalize) target = normalize_fft_results(target); // main.cpp:74-76
         logger.result_stats(validate_result(target, valid), i == 1 && print_header);
     }
     return 0;

@@ -4,6 +4,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
 from conftest import load_package
@@ -75,3 +76,46 @@ def test_argument_errors_without_a_device():
     rec = xc.LaunchRecord()
     assert lib.xcorr_last_launch(ctypes.byref(rec)) == 1
     assert b"No kernel launch" in lib.xcorr_last_error()
+
+
+def fft_module():
+    import importlib
+    return importlib.import_module(load_package().__name__ + ".fft")
+
+
+def test_fft_library_exports_every_declared_symbol():
+    fft = fft_module()
+    text = re.sub(r"/\*.*?\*/", "", open(fft.FFT_HEADER_PATH).read(), flags=re.S)
+    names = sorted(set(re.findall(r"\b(xcorr_[a-z0-9_]+)\s*\(", text)))
+    assert len(names) == 15 and "xcorr_fft_plan_forward" in names and "xcorr_scatter_f64" in names
+    if not os.path.exists(fft.FFT_LIB_PATH):
+        pytest.fail(f"{fft.FFT_LIB_PATH} not built")
+    for name in names:
+        assert hasattr(fft.lib(), name), name
+
+
+def test_fft_argument_errors_without_a_device():
+    fft = fft_module()
+    lib = fft.lib()
+    plan = ctypes.c_void_p()
+    assert lib.xcorr_fft_plan_forward(ctypes.byref(plan), 8, 8, 1, 2) == 1
+    assert b"elem" in lib.xcorr_fft_last_error()
+    assert lib.xcorr_fft_plan_forward(None, 8, 8, 1, 4) == 1
+    assert lib.xcorr_fft_plan_inverse(ctypes.byref(plan), 0, 8, 1, 4) == 1
+    dummy = ctypes.c_void_p(16)
+    assert lib.xcorr_hadamard_original_f32(dummy, dummy, 5, 8, 1, 1, 0, None) == 1
+    assert lib.xcorr_hadamard_n_to_m_over_output_f64(dummy, None, dummy, 5, 8, 1, 1, 256, 10, None) == 1
+    assert lib.xcorr_scatter_f32(dummy, dummy, 8, 8, 1, 4, 16, 0, 0, 256, 10, None) == 1  # does not fit
+    assert lib.xcorr_fft_exec_forward(None, dummy, dummy) == 1
+
+
+def test_fft_normalize_matches_the_definition():
+    """numpy mirror of fft_helpers.hpp:193-262 against scipy's full correlation."""
+    from scipy.signal import correlate2d
+    fft = fft_module()
+    rng = np.random.default_rng(5)
+    for rows, cols in [(1, 1), (4, 4), (3, 5), (6, 2), (1, 7)]:
+        a, b = rng.random((rows, cols)), rng.random((rows, cols))
+        s = (2 * rows, 2 * cols)
+        raw = np.fft.irfft2(np.fft.rfft2(a, s=s) * np.conj(np.fft.rfft2(b, s=s)), s=s) * (4 * rows * cols)
+        assert np.allclose(fft.normalize(raw[None])[0], correlate2d(a, b, mode="full"), atol=1e-12)

@@ -33,7 +33,7 @@ def gpu_names():
     from cross_cli import cross_path
 
     out = subprocess.run([cross_path(), "list"], capture_output=True, text=True).stdout.split()
-    return [n for n in out if not n.startswith("cpu_")]
+    return [n for n in out if not n.startswith(("cpu_", "fft_"))]
 
 
 @pytest.mark.parametrize("dtype", ["single", "double"])
