@@ -106,6 +106,7 @@ typedef struct xcorr_launch_record {
     unsigned rows_per_worker;  /* left rows one work item reduces over */
     unsigned distribution_type;
     unsigned uses_atomics;     /* 1: partial sums are added with float atomics into a zeroed output */
+    unsigned blocks_per_cu;    /* workgroups of this kernel one CU holds at a time (0: not recorded) */
 } xcorr_launch_record;
 
 typedef struct xcorr_device_info {

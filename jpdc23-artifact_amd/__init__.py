@@ -73,6 +73,7 @@ class LaunchRecord(ctypes.Structure):
         ("rows_per_worker", ctypes.c_uint),
         ("distribution_type", ctypes.c_uint),
         ("uses_atomics", ctypes.c_uint),
+        ("blocks_per_cu", ctypes.c_uint),
     ]
 
     def as_dict(self):

@@ -27,18 +27,16 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)); }
 
-// Relative cost of running the request on a specialisation, calibrated on MI355X sweeps of
-// 64x64 ... 1024x1024 matrices in all four modes:
+// Relative cost of running a request of the one-output-row families on one of their tiles
+// (their four wavefronts tile 2x2 over the shifts):
 //   * work issued for partial overlaps at tile edges: a wavefront skips what cannot overlap its
-//     own tile, but wavefronts that own different shift tiles of one block wait for each other
-//     after every staged band, so for those both the wavefront tile and the block tile count;
+//     own tile, but the wavefronts of a block wait for each other after every staged band, so both
+//     the wavefront tile and the block tile count;
 //   * lanes idling over matrices that do not exist;
-//   * the issue rate of the tile: one-row tiles lose issue slots to LDS reads (a read plus the
-//     wait that guards it displace about nine fp32 FMA slots, half as many fp64 ones); among
-//     the grouped tiles 8x4 measured fastest, 4x4 and 8x8 (which spills a little) about 8 % slower (fp64: 8x8 5 % slower);
-//   * lanes laid over matrices stage one band per matrix, and a right band carries a halo of
-//     TYW-1 rows: +2.8 % per extra right matrix, +2 % per extra left matrix.
-// Hints scale the cost a little so that the nearest of equally good specialisations wins.
+//   * issue slots lost to LDS reads (a read plus the wait that guards it displace about nine fp32
+//     FMA slots, half as many fp64 ones);
+//   * several matrices per lane: the register ring of right rows grows, some spills.
+// The reference's tuning integers only break ties (2 % per doubling away from the request).
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
     double waste_y = std::sqrt((double)(rq.H + s.TYW()) * (rq.H + s.TYB())) / rq.H;
@@ -46,23 +44,11 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double util_v = (double)rq.nV / ((double)ceil_div(rq.nV, s.NVB()) * s.NVB());
     double util_u = (double)nu / ((double)ceil_div(nu, s.NUB()) * s.NUB());
     double cost = waste_x * waste_y / (util_v * util_u);
-    if (s.A == 1) {
-        int vk = 16 / s.elem_bytes;
-        double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
-        double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
-        cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
-    } else if (s.A == 8 && s.B == 8) {
-        cost *= s.elem_bytes == 4 ? 1.08 : 1.05;
-    } else if (s.A == 4 && s.B == 4) {
-        cost *= s.elem_bytes == 4 ? 1.08 : 1.0;
-    }
-    cost *= 1.0 + 0.028 * (s.LU - 1) + 0.02 * (s.LV - 1);
-    if (s.NV * s.NU > 1) cost *= 1.15; // several matrices per lane: the register ring of right rows grows, some spills
-    if (s.WX * s.WY * s.WZ < 4) cost *= 1.25; // fewer than one wavefront per SIMD per block: uneven SIMD load
-    if (s.A > 1 && s.WZ == 1) cost *= 1.1; // shift-tiled blocks wait at the barriers of partial stages
-    // the reference's tuning integers were found for its own kernels on other hardware: they only
-    // break ties here (2 % per doubling away from the request)
-    if (rq.y_shifts > 1) cost *= 1.0 + 0.02 * log2_ratio(s.A, rq.y_shifts);
+    int vk = 16 / s.elem_bytes;
+    double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
+    double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
+    cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
+    if (s.NV * s.NU > 1) cost *= 1.15;
     if (rq.left_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NV * s.LV, rq.left_mats);
     if (rq.right_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NU * s.LU, rq.right_mats);
     if (rq.waves) cost *= 1.0 + 0.01 * log2_ratio(s.WX * s.WY * s.WZ, rq.waves);
@@ -86,22 +72,159 @@ static long count_chunks(const EngineSpec &s, int H, int nty, int rc, int *max_c
     return total;
 }
 
+// Fills the geometry of `plan` for specialisation `s` with the reduction over left rows cut into
+// chunks of `rc` rows (rc <= 0 or rc >= H: not cut).
+static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, EnginePlan &plan) {
+    plan.spec = &s;
+    const int Sx = 2 * rq.W - 1, Sy = 2 * rq.H - 1;
+    plan.ntx = ceil_div(Sx, s.TXB());
+    plan.nty = ceil_div(Sy, s.TYB());
+    plan.nvg = ceil_div(rq.nV, s.NVB());
+    plan.nug = ceil_div(rq.group_m > 0 ? rq.group_m : rq.nU, s.NUB());
+    int dist = rq.dist == XCORR_DIST_NONE ? 0 : rq.dist == XCORR_DIST_RECTANGLE ? 1 : rq.dist == XCORR_DIST_TRIANGLE ? 2 : -1;
+    if (rq.caller_zeroes) {
+        // split-row contract (reference one_to_one.hpp:276-288): zeroed output, atomics
+        if (dist < 0) dist = 1; // the reference's default is "rectangle" (one_to_one.hpp:232)
+        if (rc <= 0) rc = s.RL;
+        if (dist == 0) rc = rq.H;
+        plan.atomic = 1;
+        plan.zero_fill = false;
+    } else if (rc <= 0 || rc >= rq.H || !rq.may_split) {
+        rc = rq.H;
+        dist = 0;
+        plan.atomic = 0;
+        plan.zero_fill = false;
+    } else {
+        if (dist <= 0) dist = 2;
+        plan.atomic = 1;
+        plan.zero_fill = true;
+    }
+    if (rc > rq.H) rc = rq.H;
+    plan.rows_per_chunk = rc;
+    plan.dist = dist;
+
+    // workers along y: (y tile, chunk) pairs
+    int max_chunks = 0;
+    long total_chunks = count_chunks(s, rq.H, plan.nty, rc, &max_chunks);
+    if (dist == 0)
+        plan.nworkers_y = plan.nty;
+    else if (dist == 1)
+        plan.nworkers_y = plan.nty * max_chunks;
+    else
+        plan.nworkers_y = (int)total_chunks;
+    long items = (long)plan.nvg * plan.nug * plan.nworkers_y * plan.ntx;
+    if (items <= 0 || items > 0x7fffffffL) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: %ld work items are out of range", rq.family, items);
+    plan.total_items = (int)items;
+    plan.grid = (unsigned)items;
+    return XCORR_OK;
+}
+
+// Predicted run time in microseconds of a grouped-tile plan. The launch is seen as `items` blocks
+// of four wavefronts (one per SIMD) of which a CU holds `occ` at a time:
+//   * a block issues A*B FMAs per lane for every (right row, right column) its shift tile overlaps;
+//     a chunk of rc left rows meets rc + A - 1 right rows, so short chunks pay for the window;
+//   * with many blocks the run is bound by the issue rate of the CUs (average block), with few by
+//     the largest block (the centre tile, all rows and columns) at the issue rate one wavefront per
+//     SIMD reaches alone, which is less than half of what several resident wavefronts reach together;
+//     the two regimes blend: issue-bound time of all blocks plus a share of the largest block's time;
+//   * every block costs a fixed prologue / epilogue and every staged band a little; a split plan
+//     pays the clear kernel and the atomic adds of all blocks at the rate the memory system takes
+//     them (lower when the lanes of a wavefront write to different result matrices).
+// The constants were fitted to sweeps of all grouped tiles and chunk sizes over 16x16 ... 1024x1024
+// matrices and 1 ... 1024 pairs on MI355X; `issue_factor` and `stage_factor` are per tile.
+static double predict_us(const EngineSpec &s, const EngineRequest &rq, const EnginePlan &plan) {
+    const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.LV * s.LU > 1;
+    const double t_block = 3.87, e_alone = 0.415, e_full = 0.995, t_stage = 0.0839, k_tail = 0.306;
+    const double t_clear = f32 ? 1.36 : 0.0, t_atomic = f32 ? 0.0384 : 0.0186;
+    const double us_per_atomic = lanes_over_matrices ? (f32 ? 5.4e-6 : 5.1e-6) : (f32 ? 2.9e-6 : 7.2e-6);
+    const double cyc = (f32 ? 2.0 : 4.0) / 2100.0; // microseconds per FMA instruction of a wavefront
+    const double W = rq.W, H = rq.H, TXW = s.TXB(), TYW = s.TYB();
+    const bool split = plan.atomic != 0;
+    const double rc = plan.rows_per_chunk;
+    const double cols_avg = std::fmin(W, W * (W + TXW) / (plan.ntx * TXW));
+    const double rows_tile = std::fmin(H, H * (H + TYW) / (plan.nty * TYW));
+    const double rows_avg = (split ? std::fmin(rc, rows_tile) : rows_tile) + s.A - 1;
+    const double rows_max = (split ? rc : H) + s.A - 1;
+    const double per_element = (double)s.NV * s.NU * s.A * s.B / s.WZ * s.issue_factor;
+    const double inst_avg = per_element * rows_avg * cols_avg, inst_max = per_element * rows_max * W;
+    const double stages_avg = std::ceil(rows_avg / s.RL) * std::ceil((cols_avg + TXW) / s.KBX) * s.stage_factor;
+    const double stages_max = std::ceil(rows_max / s.RL) * std::ceil((W + TXW) / s.KBX) * s.stage_factor;
+    const double items = plan.total_items;
+    const int cus = device_cus(), occ = s.resident_blocks();
+    double n1 = std::ceil(items / cus);
+    if (n1 > occ) n1 = occ;
+    const double fixed = t_block + (split && !lanes_over_matrices ? t_atomic * s.A * s.B : 0.0);
+    const double crit = fixed + t_stage * stages_max + std::fmax(inst_max * cyc / e_alone, n1 * inst_max * cyc / e_full);
+    const double per_block = (fixed + t_stage * stages_avg) / n1 + inst_avg * cyc / e_full;
+    const double tail = k_tail * crit;
+    double t = std::fmax(items * per_block / cus + tail, crit);
+    if (split) t += t_clear + items * 64.0 * s.A * s.B * us_per_atomic;
+    return t;
+}
+
+// Grouped families: every compatible tile is tried with the reduction uncut and cut into 2, 3, 4, 6 ...
+// groups of G = A + 1 rows (the granule of the inner loop); the plan with the shortest predicted
+// run time wins. The reference's tuning integers only break ties (2 % per doubling away).
+static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int count, EnginePlan &plan) {
+    static const int ladder[] = {0, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+    bool found = false;
+    double best = 0;
+    for (int i = 0; i < count; ++i) {
+        const EngineSpec &s = specs[i];
+        if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
+        if (rq.group_m > 0 && s.NVB() != 1) continue;
+        if (rq.spec_index == 0) {
+            if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
+            if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
+            if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
+        }
+        const int G = s.A + 1;
+        for (int k : ladder) {
+            int rc = k * G;
+            if (rq.rows_per_worker > 0 || rq.caller_zeroes) {
+                if (k != 0) break;
+                rc = (int)rq.rows_per_worker;
+            } else if (k != 0 && (!rq.may_split || rc >= rq.H)) {
+                break;
+            } else if (k != 0 && s.LV * s.LU > 1 && (rc < 36 || rq.H < 72)) {
+                continue; // measured: short chunks of tiles whose lanes lie over matrices lose to their scattered atomic adds
+            }
+            EnginePlan cand;
+            if (int e = shape_plan(s, rq, rc, cand)) return e;
+            double t = predict_us(s, rq, cand);
+            if (rq.y_shifts > 1) t *= 1.0 + 0.02 * log2_ratio(s.A, rq.y_shifts);
+            if (rq.left_mats) t *= 1.0 + 0.02 * log2_ratio(s.NV * s.LV, rq.left_mats);
+            if (rq.right_mats) t *= 1.0 + 0.02 * log2_ratio(s.NU * s.LU, rq.right_mats);
+            if (!found || t < best) {
+                found = true;
+                best = t;
+                plan = cand;
+            }
+        }
+    }
+    if (!found)
+        return fail(XCORR_ERR_UNSUPPORTED, "%s: no compiled specialisation matches x_shifts_per_thread=%u lanes_x=%u lanes_y=%u",
+                    rq.family, rq.x_shifts, rq.lanes_x, rq.lanes_y);
+    return XCORR_OK;
+}
+
 int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     int count = 0;
     const EngineSpec *specs = rq.elem_bytes == 4 ? engine_specs_f32(&count) : engine_specs_f64(&count);
-    const EngineSpec *best = nullptr;
+    if (rq.spec_index > (unsigned)count)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %u does not exist (%d compiled)", rq.family, rq.spec_index, count);
+    if (rq.spec_index > 0 && rq.group_m > 0 && specs[rq.spec_index - 1].NVB() != 1)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %s cannot pair one left matrix with a group", rq.family,
+                    specs[rq.spec_index - 1].name);
+    const bool grouped = rq.spec_index > 0 ? specs[rq.spec_index - 1].A > 1 : rq.y_shifts != 1;
+    if (grouped) return plan_grouped(rq, specs, count, plan);
+
+    // one-output-row families: relative cost of the tile, then the split rule below
+    const EngineSpec *best = rq.spec_index > 0 ? &specs[rq.spec_index - 1] : nullptr;
     double best_cost = 0;
-    if (rq.spec_index > 0) {
-        if ((int)rq.spec_index > count)
-            return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %u does not exist (%d compiled)", rq.family, rq.spec_index, count);
-        const EngineSpec &s = specs[rq.spec_index - 1];
-        if (rq.group_m > 0 && s.NVB() != 1)
-            return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %s cannot pair one left matrix with a group", rq.family, s.name);
-        best = &s;
-    }
     for (int i = 0; i < count && rq.spec_index == 0; ++i) {
         const EngineSpec &s = specs[i];
-        if ((rq.y_shifts == 1) != (s.A == 1)) continue; // one-output-row families vs grouped families
+        if (s.A != 1) continue;
         if (rq.group_m > 0 && s.NVB() != 1) continue;
         if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
         if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
@@ -115,77 +238,30 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     if (!best)
         return fail(XCORR_ERR_UNSUPPORTED, "%s: no compiled specialisation matches x_shifts_per_thread=%u lanes_x=%u lanes_y=%u",
                     rq.family, rq.x_shifts, rq.lanes_x, rq.lanes_y);
-    plan.spec = best;
-    const int Sx = 2 * rq.W - 1, Sy = 2 * rq.H - 1;
-    plan.ntx = ceil_div(Sx, best->TXB());
-    plan.nty = ceil_div(Sy, best->TYB());
-    plan.nvg = ceil_div(rq.nV, best->NVB());
-    plan.nug = ceil_div(rq.group_m > 0 ? rq.group_m : rq.nU, best->NUB());
-    const long tiles = (long)plan.ntx * plan.nty * plan.nvg * plan.nug;
-
-    int dist = rq.dist == XCORR_DIST_NONE ? 0 : rq.dist == XCORR_DIST_RECTANGLE ? 1 : rq.dist == XCORR_DIST_TRIANGLE ? 2 : -1;
     int rc = (int)rq.rows_per_worker;
-    if (rq.caller_zeroes) {
-        // split-row contract (reference one_to_one.hpp:276-288): zeroed output, atomics
-        if (dist < 0) dist = 1; // the reference's default is "rectangle" (one_to_one.hpp:232)
-        if (rc <= 0) rc = best->RL;
-        if (dist == 0) rc = rq.H;
-        plan.atomic = 1;
-        plan.zero_fill = false;
-    } else {
-        // Few tiles, or long ones: cut the reduction over left rows into chunks (whole groups of
-        // G = A+1 rows, the granule of the inner loop) until the launch has about 128 work items
-        // per CU. Finer items even out the last wave of blocks and cost little, because the four
-        // wavefronts of a block add their partial tiles in LDS before the atomic adds (1024x1024:
-        // flat between 18 and 54 rows, 3 % slower at 72, 6 % at 144; 2048x2048 unsplit 20 % slower).
-        // Items shorter than 20 rows only pay for tiny problems that would otherwise leave CUs
-        // without work. Lanes laid over matrices write one result matrix per lane: their
-        // atomics would not coalesce, so such tiles are never split by the planner itself.
-        const bool split_ok = rq.may_split && best->LV * best->LU == 1;
+    if (!rq.caller_zeroes && rc <= 0 && rq.may_split) {
+        // Few tiles, or long ones: cut the reduction over left rows into chunks of whole groups until
+        // the launch has about 128 work items per CU; items shorter than 20 rows only pay for tiny
+        // problems that would otherwise leave CUs without work.
+        EnginePlan whole;
+        if (int e = shape_plan(*best, rq, 0, whole)) return e;
+        const long tiles = whole.total_items;
         const int G = best->A + 1;
         const int rc_most = 4 * best->RL;
-        if (rc <= 0 && split_ok && (tiles < 48L * device_cus() || rq.H > rc_most)) {
+        if (tiles < 48L * device_cus() || rq.H > rc_most) {
             const long target = 128L * device_cus();
-            const long per_tile_column = (long)plan.ntx * plan.nvg * plan.nug;
-            // shortest item: 20 rows, or 9 when that leaves CUs without work (rounded up to whole groups)
+            const long per_tile_column = (long)whole.ntx * whole.nvg * whole.nug;
             const int k_normal = ceil_div(20, G), k_tiny = ceil_div(9, G);
-            const int k_min = per_tile_column * count_chunks(*best, rq.H, plan.nty, k_normal * G, nullptr) < 2L * device_cus() ? k_tiny : k_normal;
+            const int k_min = per_tile_column * count_chunks(*best, rq.H, whole.nty, k_normal * G, nullptr) < 2L * device_cus() ? k_tiny : k_normal;
             int k = (rq.H < rc_most ? rq.H : rc_most) / G;
             for (; k >= k_min; --k) {
                 rc = k * G;
-                if (per_tile_column * count_chunks(*best, rq.H, plan.nty, rc, nullptr) >= target) break;
+                if (per_tile_column * count_chunks(*best, rq.H, whole.nty, rc, nullptr) >= target) break;
             }
             if (rc <= 0) rc = rq.H;
         }
-        if (rc <= 0 || rc >= rq.H || !rq.may_split) {
-            rc = rq.H;
-            dist = 0;
-            plan.atomic = 0;
-            plan.zero_fill = false;
-        } else {
-            if (dist <= 0) dist = 2;
-            plan.atomic = 1;
-            plan.zero_fill = true;
-        }
     }
-    if (rc > rq.H) rc = rq.H;
-    plan.rows_per_chunk = rc;
-    plan.dist = dist;
-
-    // workers along y: (y tile, chunk) pairs
-    int max_chunks = 0;
-    long total_chunks = count_chunks(*best, rq.H, plan.nty, rc, &max_chunks);
-    if (dist == 0)
-        plan.nworkers_y = plan.nty;
-    else if (dist == 1)
-        plan.nworkers_y = plan.nty * max_chunks;
-    else
-        plan.nworkers_y = (int)total_chunks;
-    long items = (long)plan.nvg * plan.nug * plan.nworkers_y * plan.ntx;
-    if (items <= 0 || items > 0x7fffffffL) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: %ld work items are out of range", rq.family, items);
-    plan.total_items = (int)items;
-    plan.grid = (unsigned)items;
-    return XCORR_OK;
+    return shape_plan(*best, rq, rc, plan);
 }
 
 template <typename T>
@@ -246,6 +322,7 @@ int run_engine(const EngineRequest &rq, hipStream_t stream) {
     rec.rows_per_worker = plan.rows_per_chunk;
     rec.distribution_type = plan.dist == 0 ? XCORR_DIST_NONE : plan.dist == 1 ? XCORR_DIST_RECTANGLE : XCORR_DIST_TRIANGLE;
     rec.uses_atomics = plan.atomic;
+    rec.blocks_per_cu = plan.spec->resident_blocks();
     have_last_launch() = true;
     return XCORR_OK;
 }

@@ -23,6 +23,12 @@ struct EngineSpec {
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
     hipError_t (*launch)(const void *args, unsigned grid, hipStream_t stream);
+    // workgroups of this kernel that one CU holds at a time (registers and LDS), asked of the runtime once
+    int (*resident_blocks)();
+    // calibration of the planner's run-time model for grouped tiles: FMA issue slots a wavefront spends per
+    // useful FMA instruction (LDS reads, waits and address arithmetic included), and the relative cost
+    // of staging one band
+    double issue_factor, stage_factor;
     int TXW() const { return LX * B; }
     int TYW() const { return LY * A; }
     int TXB() const { return TXW() * WX; }
@@ -32,8 +38,7 @@ struct EngineSpec {
 };
 
 template <class C>
-hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
-    using T = typename C::value_type;
+hipError_t allow_large_lds() {
     static bool attr_set = false;
     if (!attr_set && C::LDS_BYTES > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&engine_kernel<C>),
@@ -41,12 +46,34 @@ hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
         if (e != hipSuccess) return e;
         attr_set = true;
     }
+    return hipSuccess;
+}
+
+template <class C>
+hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
+    using T = typename C::value_type;
+    if (hipError_t e = allow_large_lds<C>(); e != hipSuccess) return e;
     engine_kernel<C><<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
     return hipGetLastError();
 }
 
 template <class C>
-constexpr EngineSpec make_spec(const char *name) {
+int resident_blocks_engine() {
+    static int blocks = 0;
+    if (blocks == 0) {
+        int n = 0;
+        if (allow_large_lds<C>() != hipSuccess ||
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(&engine_kernel<C>), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
+            (void)hipGetLastError();
+            n = 1;
+        }
+        blocks = n;
+    }
+    return blocks;
+}
+
+template <class C>
+constexpr EngineSpec make_spec(const char *name, double issue_factor = 1.0, double stage_factor = 1.0) {
     return EngineSpec{name,   (int)sizeof(typename C::value_type),
                       C::A,   C::B,
                       C::K,   C::NV,
@@ -56,7 +83,7 @@ constexpr EngineSpec make_spec(const char *name) {
                       C::WY,  C::RL,
                       C::KBX, C::WZ,
                       C::LDS_BYTES,
-                      C::NT,  &launch_engine<C>};
+                      C::NT,  &launch_engine<C>, &resident_blocks_engine<C>, issue_factor, stage_factor};
 }
 
 // defined in engine_f32.hip / engine_f64.hip

@@ -266,7 +266,7 @@ def test_every_compiled_specialisation_by_index(oracle):
         assert len(names) >= 9
 
 
-def test_launch_record_and_errors():
+def test_launch_record_and_errors(oracle):
     xc = load_package()
     rng = np.random.default_rng(700)
     left = ints(rng, (32, 32), np.float32)
@@ -275,10 +275,18 @@ def test_launch_record_and_errors():
     say(rec)
     assert rec["kernel"].startswith("grouped_overlap/")
     assert rec["y_shifts_per_thread"] in (4, 8) and rec["block"][0] % 64 == 0 and rec["grid"][0] >= 1
+    assert 1 <= rec["blocks_per_cu"] <= 16  # occupancy the planner's run-time model works with
     # the geometry fields select a tile exactly
     xc.run("grouped_overlap", left, left, 1, params=xc.make_params(x_shifts_per_thread=8, lanes_x=8, lanes_y=8))
     rec = xc.last_launch()
     assert rec["x_shifts_per_thread"] == 8 and rec["lanes_x"] == 8 and rec["lanes_y"] == 8
+    # the planner cuts the reduction of a small multi-matrix problem into chunks (atomic adds into an output it
+    # clears itself) also for tiles whose lanes lie over matrices; an explicit rows_per_thread is taken as it is
+    one, many = ints(rng, (1, 96, 96), np.float32), ints(rng, (8, 96, 96), np.float32)
+    got = xc.run("multimat_right_grouped", one, many, 8, n_left=1, n_right=8, params=xc.make_params(specialisation=14, rows_per_thread=36))
+    rec = xc.last_launch()
+    assert rec["lanes_right"] == 8 and rec["uses_atomics"] == 1 and rec["rows_per_worker"] == 36
+    np.testing.assert_array_equal(got, oracle.one_to_many(one, many))
     with pytest.raises(xc.XcorrError, match="Too many shifts per thread"):
         xc.run("grouped_overlap", left, left, 1, params=xc.make_params(shifts_per_thread=9))
     with pytest.raises(xc.XcorrError, match="Too many warps"):
@@ -286,3 +294,31 @@ def test_launch_record_and_errors():
     info = xc.device_info()
     say(info.name, info.arch, info.compute_units, info.clock_khz, info.fp32_vector_peak_tflops)
     assert b"gfx950" in info.arch
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_planner_choices_for_few_matrices_of_medium_size(oracle, dtype):
+    """Problems with too few tiles to fill the GPU: the planner's run-time model cuts the reduction over
+    left rows into chunks (atomic adds into an output it clears itself), also for tiles whose lanes lie
+    over matrices, or falls back to the small tile. Whatever it picks, integer-valued inputs must match
+    the oracle exactly; the plan is printed."""
+    xc = load_package()
+    rng = np.random.default_rng(800)
+    for family, mode, n_left, n_right, shape in [("multimat_right_grouped", "one_to_many", 1, 32, (96, 80)),
+                                                 ("multimat_right_grouped", "one_to_many", 1, 8, (128, 128)),
+                                                 ("multimat_both_grouped", "n_to_m", 4, 8, (96, 96)),
+                                                 ("multimat_both_grouped", "n_to_m", 16, 16, (40, 24))]:
+        left = ints(rng, (n_left,) + shape, dtype)
+        right = ints(rng, (n_right,) + shape, dtype)
+        n_out = n_left * n_right if mode == "n_to_m" else n_right
+        exp = getattr(oracle, mode)(left, right, threads=8)
+        for kw in ({}, dict(rows_per_thread=27), dict(rows_per_thread=1000)):
+            got = xc.run(family, left, right, n_out, n_left=n_left, n_right=n_right, params=xc.make_params(**kw))
+            rec = xc.last_launch()
+            say(mode, np.dtype(dtype).name, n_left, n_right, shape, kw, rec["kernel"], "rows", rec["rows_per_worker"], "grid", rec["grid"][0],
+                "atomics", rec["uses_atomics"])
+            if kw.get("rows_per_thread") == 27:
+                assert rec["rows_per_worker"] == 27 and rec["uses_atomics"] == 1
+            if kw.get("rows_per_thread") == 1000:
+                assert rec["rows_per_worker"] == shape[0] and rec["uses_atomics"] == 0
+            check(got, exp, True, f"{mode} {n_left}x{n_right} {shape} {kw}")
