@@ -164,7 +164,7 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
 
 // Grouped families: every compatible tile is tried with the reduction uncut and cut into 2, 3, 4, 6 ...
 // groups of G = A + 1 rows (the granule of the inner loop); the plan with the shortest predicted
-// run time wins. The reference's tuning integers only break ties (2 % per doubling away).
+// run time wins. The reference's tuning integers only break ties (0.5 % per doubling away).
 static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int count, EnginePlan &plan) {
     static const int ladder[] = {0, 2, 3, 4, 6, 8, 12, 16, 24, 32};
     bool found = false;
@@ -192,9 +192,9 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
             EnginePlan cand;
             if (int e = shape_plan(s, rq, rc, cand)) return e;
             double t = predict_us(s, rq, cand);
-            if (rq.y_shifts > 1) t *= 1.0 + 0.02 * log2_ratio(s.A, rq.y_shifts);
-            if (rq.left_mats) t *= 1.0 + 0.02 * log2_ratio(s.NV * s.LV, rq.left_mats);
-            if (rq.right_mats) t *= 1.0 + 0.02 * log2_ratio(s.NU * s.LU, rq.right_mats);
+            if (rq.y_shifts > 1) t *= 1.0 + 0.005 * log2_ratio(s.A, rq.y_shifts);
+            if (rq.left_mats) t *= 1.0 + 0.005 * log2_ratio(s.NV * s.LV, rq.left_mats);
+            if (rq.right_mats) t *= 1.0 + 0.005 * log2_ratio(s.NU * s.LU, rq.right_mats);
             if (!found || t < best) {
                 found = true;
                 best = t;
