@@ -87,7 +87,9 @@ typedef struct xcorr_params {
     unsigned strided_load;                   /* load pattern of the reference's staging; no effect here */
     unsigned column_group_per_block;         /* 1: one block per group of 64 columns, sums added atomically (caller zeroes `out`) */
     unsigned block_size;                     /* block-per-overlap: threads per block, 0 = 128, <= 1024 */
-    unsigned reserved[2];
+    unsigned column_chunks;                  /* grouped families: cut the reduction over right columns into this many chunks
+                                                (atomic adds, like rows_per_thread for rows); 0 = planner decides, no counterpart in the reference */
+    unsigned reserved;
 } xcorr_params;
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the
@@ -107,6 +109,7 @@ typedef struct xcorr_launch_record {
     unsigned distribution_type;
     unsigned uses_atomics;     /* 1: partial sums are added with float atomics into a zeroed output */
     unsigned blocks_per_cu;    /* workgroups of this kernel one CU holds at a time (0: not recorded) */
+    unsigned column_chunks;    /* chunks the reduction over right columns is cut into (1: not cut) */
 } xcorr_launch_record;
 
 typedef struct xcorr_device_info {

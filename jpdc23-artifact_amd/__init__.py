@@ -50,7 +50,8 @@ class Params(ctypes.Structure):
         ("strided_load", ctypes.c_uint),
         ("column_group_per_block", ctypes.c_uint),
         ("block_size", ctypes.c_uint),
-        ("reserved", ctypes.c_uint * 2),
+        ("column_chunks", ctypes.c_uint),
+        ("reserved", ctypes.c_uint),
     ]
 
 
@@ -74,6 +75,7 @@ class LaunchRecord(ctypes.Structure):
         ("distribution_type", ctypes.c_uint),
         ("uses_atomics", ctypes.c_uint),
         ("blocks_per_cu", ctypes.c_uint),
+        ("column_chunks", ctypes.c_uint),
     ]
 
     def as_dict(self):

@@ -47,7 +47,9 @@ struct EngineArgs {
     int ntx, nty;       // number of block tiles in x and y
     int nworkers_y;     // number of (y tile, chunk) workers
     int nvg, nug;       // left / right matrix groups
-    int total_items;    // nvg * nug * nworkers_y * ntx
+    int total_items;    // nvg * nug * nworkers_y * ntx * x_chunks
+    int x_chunks;       // >1: the right columns a tile overlaps are cut into chunks of x_chunk_cols (atomic adds)
+    int x_chunk_cols;   // multiple of K * WZ
 };
 
 // WZ_ > 1: the WZ_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
@@ -385,6 +387,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     // ---- decode the work item (uniform over the threads that share it) ----
     int item = (int)blockIdx.x;
     if (item >= g.total_items) return;
+    const int xch = item % g.x_chunks;
+    item /= g.x_chunks;
     const int mat = item % (g.nvg * g.nug);
     item /= (g.nvg * g.nug);
     const int rc = g.rows_per_chunk;
@@ -445,6 +449,16 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     xr_lo = (xr_lo / C::KBX) * C::KBX;
     int xr_hi = W - sxb;
     if (xr_hi > W) xr_hi = W;
+    // this work item's chunk of those columns
+    int col_lo = 0, col_hi = W;
+    if (g.x_chunks > 1) {
+        col_lo = xr_lo + xch * g.x_chunk_cols;
+        col_hi = col_lo + g.x_chunk_cols;
+        if (col_hi > xr_hi) col_hi = xr_hi;
+        if (col_lo >= col_hi) return; // the tile overlaps fewer columns than the widest one
+        xr_lo = (col_lo / C::KBX) * C::KBX;
+        xr_hi = col_hi;
+    }
 
     // ---- lane coordinates ----
     const int lane = tid & 63;
@@ -533,6 +547,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             if (W - 1 - x0 < lim) lim = W - 1 - x0;
             int h = lim < 0 ? 0 : lim / K + 1;
             if (h < kc_hi) kc_hi = h;
+        }
+        if (g.x_chunks > 1) {
+            const int lo = (col_lo - x0) / K, hi = (col_hi - x0 + K - 1) / K; // col_lo - x0 is a multiple of K or negative
+            if (col_lo > x0 && lo > kc_lo) kc_lo = lo;
+            if (hi < kc_hi) kc_hi = hi;
         }
         if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
         if (jj_lo < jj_hi || (jj_lo == jj_hi && tail > 0))

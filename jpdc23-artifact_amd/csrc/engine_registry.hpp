@@ -102,6 +102,7 @@ struct EngineRequest {
     unsigned y_shifts, x_shifts, left_mats, right_mats, lanes_x, lanes_y, waves;
     unsigned spec_index;      // 1-based: use exactly this entry of the specialisation table
     unsigned rows_per_worker; // 0 = planner decides
+    unsigned column_chunks;   // 0 = planner decides (grouped families only)
     unsigned dist;            // XCORR_DIST_*
     bool caller_zeroes;       // true: split-row contract, output arrives zeroed, always accumulate atomically
     bool may_split;           // planner may split the reduction and clear the output itself
@@ -111,6 +112,7 @@ struct EnginePlan {
     const EngineSpec *spec;
     int ntx, nty, nworkers_y, nvg, nug;
     int rows_per_chunk, dist, atomic, total_items;
+    int x_chunks, x_chunk_cols; // chunks of right columns per tile (1: not cut) and their width
     bool zero_fill;
     unsigned grid;
 };

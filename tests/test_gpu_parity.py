@@ -322,3 +322,33 @@ def test_planner_choices_for_few_matrices_of_medium_size(oracle, dtype):
             if kw.get("rows_per_thread") == 1000:
                 assert rec["rows_per_worker"] == shape[0] and rec["uses_atomics"] == 0
             check(got, exp, True, f"{mode} {n_left}x{n_right} {shape} {kw}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_reduction_cut_over_columns(oracle, dtype):
+    """column_chunks cuts the reduction over right columns into work items that add atomically (on top of, or
+    instead of, the cut over left rows); every grouped tile, more chunks than columns allow, ragged widths."""
+    xc = load_package()
+    rng = np.random.default_rng(900)
+    n_specs = 14 if dtype == np.float32 else 12
+    first_grouped = 4 if dtype == np.float32 else 3
+    for family, mode, n_left, n_right, shape in [("grouped_overlap", "one_to_one", 1, 1, (40, 70)),
+                                                 ("multimat_right_grouped", "one_to_many", 1, 5, (33, 18)),
+                                                 ("multimat_both_grouped", "n_to_m", 3, 4, (21, 47))]:
+        left = ints(rng, (n_left,) + shape, dtype)
+        right = ints(rng, (n_right,) + shape, dtype)
+        n_out = n_left * n_right if mode == "n_to_m" else n_right
+        exp = getattr(oracle, mode)(left, right)
+        for spec in range(first_grouped, n_specs + 1):
+            for chunks, rows in [(2, 0), (3, 9), (8, 1000), (64, 0)]:
+                got = xc.run(family, left, right, n_out, n_left=n_left, n_right=n_right,
+                             params=xc.make_params(specialisation=spec, column_chunks=chunks, rows_per_thread=rows))
+                rec = xc.last_launch()
+                say(mode, np.dtype(dtype).name, shape, "spec", spec, rec["kernel"], "column chunks", rec["column_chunks"], "rows", rec["rows_per_worker"],
+                    "grid", rec["grid"][0])
+                assert rec["uses_atomics"] == 1 and 2 <= rec["column_chunks"] <= chunks
+                check(got, exp, True, f"{mode} spec {spec} chunks {chunks} rows {rows}")
+        # left to the planner, small problems are cut over columns too
+        got = xc.run(family, left, right, n_out, n_left=n_left, n_right=n_right)
+        say(mode, "planner", xc.last_launch())
+        check(got, exp, True, f"{mode} planner")
