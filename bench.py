@@ -77,6 +77,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel on 256 MiB so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the same run can be scaled to bytes")
+    ap.add_argument("--graph-replay", type=int, default=0, metavar="N",
+                    help="additionally capture N steps into one HIP graph and time its replays (reported under \"graph_replay\")")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (every output element is an independent reduction; "
@@ -148,6 +150,40 @@ def main():
     ev_ms = start.elapsed_ms(stop)
     rec = xc.last_launch()
 
+    graph_replay = None
+    if args.graph_replay > 0:
+        # launch-bound workloads: N steps recorded once, replayed as one submission
+        import ctypes
+
+        stream = xc.Stream()
+
+        def step_on(s):
+            if zero_first:
+                code = xc.lib().xcorr_clear_async(d_out.ptr, ctypes.c_size_t(d_out.nbytes), s)
+                assert code == 0, xc.lib().xcorr_last_error()
+            xc.launch(family, d_left, d_right, d_out, cols, rows, n_left, n_right, dtype, params, s)
+
+        step_on(stream.ptr)
+        stream.sync()
+        graph = xc.Graph(stream)
+        graph.begin()
+        for _ in range(args.graph_replay):
+            step_on(stream.ptr)
+        graph.end()
+        for _ in range(3):
+            graph.launch()
+        stream.sync()
+        replays = max(1, args.steps // 2)
+        g0 = time.perf_counter()
+        for _ in range(replays):
+            graph.launch()
+        stream.sync()
+        g_wall = time.perf_counter() - g0
+        graph_replay = {"steps_per_graph": args.graph_replay, "replays": replays,
+                        "us_per_step": round(g_wall * 1e6 / (replays * args.graph_replay), 3)}
+        graph.destroy()
+        stream.destroy()
+
     ms_per_step = wall * 1e3 / args.steps
     kernel_ms = ev_ms / args.steps
     fmas = workloads.fma_count(cfg)
@@ -194,6 +230,8 @@ def main():
         },
     }
 
+    if graph_replay:
+        result["graph_replay"] = graph_replay
     if not args.no_cpu:
         oracle = load_oracle()
         base, (lo, hi, band) = cpu_baseline(oracle, cfg, left, right)

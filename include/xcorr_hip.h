@@ -151,6 +151,17 @@ int xcorr_stream_create(void **stream);
 int xcorr_stream_destroy(void *stream);
 int xcorr_stream_sync(void *stream);
 int xcorr_device_sync(void);
+/* ---- HIP graphs: launch-bound sequences (many small instances) are captured once and replayed.
+ * No counterpart in the reference. Every entry point above may be called on a capturing stream
+ * (after one eager call of the same family and element type, so that one-time set-up is not
+ * captured); clear buffers with xcorr_clear_async (a kernel), not xcorr_memset_async, inside a
+ * capture. The stream must not be the NULL stream. ---- */
+int xcorr_clear_async(void *dev_ptr, size_t bytes, void *stream); /* bytes: multiple of 4 */
+int xcorr_graph_capture_begin(void *stream);
+int xcorr_graph_capture_end(void *stream, void **graph_exec);
+int xcorr_graph_launch(void *graph_exec, void *stream);
+int xcorr_graph_destroy(void *graph_exec);
+
 int xcorr_event_create(void **event);
 int xcorr_event_record(void *event, void *stream);
 int xcorr_event_sync(void *event);

@@ -215,6 +215,44 @@ class Event:
             pass
 
 
+class Stream:
+    """A HIP stream of default priority, owned through the C ABI."""
+
+    def __init__(self):
+        self.ptr = ctypes.c_void_p()
+        _check(lib().xcorr_stream_create(ctypes.byref(self.ptr)))
+
+    def sync(self):
+        _check(lib().xcorr_stream_sync(self.ptr))
+
+    def destroy(self):
+        if self.ptr:
+            lib().xcorr_stream_destroy(self.ptr)
+            self.ptr = ctypes.c_void_p()
+
+
+class Graph:
+    """Launches captured from a stream between begin() and end(), replayed with launch()."""
+
+    def __init__(self, stream):
+        self.stream = stream
+        self.exec = ctypes.c_void_p()
+
+    def begin(self):
+        _check(lib().xcorr_graph_capture_begin(self.stream.ptr))
+
+    def end(self):
+        _check(lib().xcorr_graph_capture_end(self.stream.ptr, ctypes.byref(self.exec)))
+
+    def launch(self, stream=None):
+        _check(lib().xcorr_graph_launch(self.exec, (stream or self.stream).ptr))
+
+    def destroy(self):
+        if self.exec:
+            lib().xcorr_graph_destroy(self.exec)
+            self.exec = ctypes.c_void_p()
+
+
 def make_params(**kw):
     p = Params()
     for k, v in kw.items():

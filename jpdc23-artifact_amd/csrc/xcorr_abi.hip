@@ -115,6 +115,44 @@ int xcorr_stream_sync(void *stream) {
     XCORR_HIP(hipStreamSynchronize(as_stream(stream)));
     return XCORR_OK;
 }
+int xcorr_clear_async(void *dev_ptr, size_t bytes, void *stream) {
+    if (!dev_ptr) return fail(XCORR_ERR_INVALID_ARGUMENT, "null device pointer");
+    if (bytes % 4 != 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "xcorr_clear_async: %zu bytes are not a multiple of 4", bytes);
+    const size_t n = bytes / 4;
+    if (n == 0) return XCORR_OK;
+    size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
+    if (blocks > 65536) blocks = 65536;
+    zero_fill_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, as_stream(stream)>>>(static_cast<float *>(dev_ptr), n);
+    XCORR_HIP(hipGetLastError());
+    return XCORR_OK;
+}
+int xcorr_graph_capture_begin(void *stream) {
+    if (!stream) return fail(XCORR_ERR_INVALID_ARGUMENT, "the NULL stream cannot be captured");
+    // relaxed: one-time set-up calls of a first launch (function attributes, occupancy queries) do not break the capture
+    XCORR_HIP(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+    return XCORR_OK;
+}
+int xcorr_graph_capture_end(void *stream, void **graph_exec) {
+    if (!stream || !graph_exec) return fail(XCORR_ERR_INVALID_ARGUMENT, "null pointer");
+    hipGraph_t graph = nullptr;
+    XCORR_HIP(hipStreamEndCapture(as_stream(stream), &graph));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    XCORR_HIP(e);
+    *graph_exec = exec;
+    return XCORR_OK;
+}
+int xcorr_graph_launch(void *graph_exec, void *stream) {
+    if (!graph_exec) return fail(XCORR_ERR_INVALID_ARGUMENT, "null graph");
+    XCORR_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+    return XCORR_OK;
+}
+int xcorr_graph_destroy(void *graph_exec) {
+    if (!graph_exec) return XCORR_OK;
+    XCORR_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+    return XCORR_OK;
+}
 int xcorr_device_sync(void) {
     XCORR_HIP(hipDeviceSynchronize());
     XCORR_HIP(hipGetLastError());
