@@ -168,3 +168,46 @@ def test_c2_band_against_oracle(oracle):
           f"max_abs={s32.max_abs:.3e} max_rel={s32.max_rel:.3e}", flush=True)
     print(f"one accumulator per element vs fp64-accumulated: rel_frobenius={s64.rel_frobenius:.3e} max_abs={s64.max_abs:.3e}", flush=True)
     assert s32.rel_frobenius <= 1e-5
+
+
+def test_output_larger_than_2_32_elements(oracle):
+    """n_to_m 130 x 128 matrices of 256x256 fp32: 16 640 results of 511x511 = 4.345e9 elements (17.4 GB), more than
+    32-bit element indices reach (the reference's dsize_t is uint32, types.cuh:12; its largest published run, 128 x 128,
+    stays 0.4 % below 2^32). Integer-valued inputs; the first, a middle and the last pairs - the last ones lie wholly
+    beyond element 2^32 - must match the oracle exactly, and the centre element of every 1000th result must equal
+    the plain dot product."""
+    import ctypes
+
+    xc = load_package()
+    rng = np.random.default_rng(77)
+    n_left, n, size = 130, 128, 256
+    left = rng.integers(-2, 3, size=(n_left, size, size)).astype(np.float32)
+    right = rng.integers(-2, 3, size=(n, size, size)).astype(np.float32)
+    per = (2 * size - 1) ** 2
+    total = n_left * n * per
+    assert total > 2 ** 32
+    d_left, d_right = xc.DeviceBuffer.from_numpy(left), xc.DeviceBuffer.from_numpy(right)
+    d_out = xc.DeviceBuffer(total * 4)
+    d_out.fill_bytes(0x7F)
+    print("n_to_m 130x128 256x256 fp32, output bytes", total * 4, flush=True)
+    xc.launch("multimat_both_grouped", d_left, d_right, d_out, size, size, n_left, n, np.float32, None)
+    xc.sync()
+    print(xc.last_launch(), flush=True)
+
+    def fetch(pair):
+        host = np.empty((2 * size - 1, 2 * size - 1), np.float32)
+        src = ctypes.c_void_p(d_out.ptr.value + pair * per * 4)
+        assert xc.lib().xcorr_memcpy_d2h(host.ctypes.data_as(ctypes.c_void_p), src, ctypes.c_size_t(host.nbytes)) == 0
+        return host
+
+    for l, r in [(0, 0), (61, 77), (128, 64), (128, 70), (129, 127)]:
+        pair = l * n + r
+        assert l < 128 or r == 64 or pair * per > 2 ** 32  # pair (128, 64) straddles element 2^32
+        got = fetch(pair)
+        exp = oracle.one_to_one(left[l], right[r], threads=8)[0]
+        np.testing.assert_array_equal(got, exp, err_msg=f"pair {l},{r}")
+    for pair in range(0, n_left * n, 1000):
+        l, r = divmod(pair, n)
+        centre = fetch(pair)[size - 1, size - 1]
+        assert centre == float(np.sum(left[l].astype(np.float64) * right[r])), pair
+    d_out.free()
