@@ -51,7 +51,10 @@ __device__ __forceinline__ void atomic_add_simple(double *p, double v) { unsafeA
 
 // ------------------------------------------------------------------ overlap-wise
 // Thread (x, y) of the strip of n_left result matrices laid side by side computes one
-// shift, for every one of the `batch` right matrices paired with its left matrix.
+// shift; blockIdx.z walks the `batch` right matrices paired with its left matrix. The products
+// are added in the order of the definition (row by row, left to right, one accumulator), so a
+// result equals the host loop's bit for bit when that is compiled with the same contraction;
+// eight element pairs are loaded ahead of the eight dependent FMAs so that the loads overlap.
 template <typename T>
 __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__ left, const T *__restrict__ right,
                                                             T *__restrict__ out, int W, int H, int n_left, int batch) {
@@ -66,14 +69,25 @@ __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__
     const int yl_lo = sy > 0 ? sy : 0, yl_hi = H + sy < H ? H + sy : H;
     const size_t in_area = (size_t)W * H, out_area = (size_t)Sx * Sy;
     const T *l = left + region * in_area;
-    for (int b = 0; b < batch; ++b) {
+    for (int b = blockIdx.z; b < batch; b += gridDim.z) {
         const size_t mat = (size_t)b * n_left + region;
         const T *r = right + mat * in_area;
         T sum = T(0);
         for (int yl = yl_lo; yl < yl_hi; ++yl) {
             const T *lrow = l + (size_t)yl * W;
             const T *rrow = r + (size_t)(yl - sy) * W - sx;
-            for (int xl = xl_lo; xl < xl_hi; ++xl) sum += rrow[xl] * lrow[xl];
+            int xl = xl_lo;
+            for (; xl + 8 <= xl_hi; xl += 8) {
+                T a[8], c[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    a[i] = rrow[xl + i];
+                    c[i] = lrow[xl + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) sum += a[i] * c[i];
+            }
+            for (; xl < xl_hi; ++xl) sum += rrow[xl] * lrow[xl];
         }
         out[mat * out_area + (size_t)oy * Sx + ox] = sum;
     }
@@ -89,7 +103,7 @@ int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsig
     dim3 block(64, 4);
     unsigned long long strip = (unsigned long long)Sx * n_left;
     if (strip > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "strip of %u result matrices is too wide", n_left);
-    dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y);
+    dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y, batch < 65535 ? batch : 65535);
     overlap_wise_kernel<T><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch);
     XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
@@ -219,12 +233,39 @@ __global__ __launch_bounds__(1024) void warp_per_overlap_kernel(const T *__restr
         }
         sum = ((part_sum[0] + part_sum[1]) + (part_sum[2] + part_sum[3])) + ((part_sum[4] + part_sum[5]) + (part_sum[6] + part_sum[7]));
     } else if (oh > 0 && ow > 0) {
-        const unsigned total = (unsigned)ow * (unsigned)oh;
-        for (unsigned i = lane; i < total; i += 64) {
-            const unsigned row = i / (unsigned)ow, col = i - row * (unsigned)ow;
-            const int yr = yr_lo + (int)row, xr = xr_lo + (int)col;
-            sum += left[(size_t)(yr + sy) * W + (xr + sx)] * right[(size_t)yr * W + xr];
+        // lanes stride the flattened overlap. Four strides are in flight with a partial sum each, and a
+        // position's (row, column) advances by 256 elements with one compare instead of a division.
+        const unsigned uow = (unsigned)ow, total = uow * (unsigned)oh;
+        const unsigned step_rows = 256u / uow, step_cols = 256u % uow;
+        T part_sum[4];
+        unsigned row[4], col[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            part_sum[k] = T(0);
+            row[k] = ((unsigned)lane + 64u * k) / uow;
+            col[k] = ((unsigned)lane + 64u * k) - row[k] * uow;
         }
+        auto product = [&](int k) {
+            const int yr = yr_lo + (int)row[k], xr = xr_lo + (int)col[k];
+            return left[(size_t)(yr + sy) * W + (xr + sx)] * right[(size_t)yr * W + xr];
+        };
+        unsigned i = (unsigned)lane;
+        for (; i + 192u < total; i += 256u) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                part_sum[k] += product(k);
+                row[k] += step_rows;
+                col[k] += step_cols;
+                if (col[k] >= uow) {
+                    col[k] -= uow;
+                    ++row[k];
+                }
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < 3; ++k)
+            if (i + 64u * k < total) part_sum[k] += product(k);
+        sum = (part_sum[0] + part_sum[1]) + (part_sum[2] + part_sum[3]);
     }
     sum = wave_sum_to_lane63(sum);
     if (lane == 63) {
