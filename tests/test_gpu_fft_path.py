@@ -126,3 +126,20 @@ def test_fft_common_steps_and_input_errors(tmp_path):
     assert rc == 3 and "expected one left matrix" in err
     rc, _, err = run_cross("run", "fft_orig_n_to_mn", rp, lp, cwd=tmp_path)
     assert rc == 3 and "not divisible" in err
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_fft_path_agrees_with_definition_kernels_at_256(dtype):
+    """Two independent device paths on the same inputs at a size the CPU oracle needs minutes for: one-to-many
+    1 x 8 matrices of 256x256, hipFFT path against the grouped definition-based kernels. Relative to the largest
+    result element: 2e-5 in fp32 (both paths round differently), 1e-11 in fp64."""
+    xc = load_package()
+    fft = fft_module()
+    rng = np.random.default_rng(48)
+    left = rng.random((1, 256, 256)).astype(dtype)
+    right = rng.random((8, 256, 256)).astype(dtype)
+    by_definition = xc.run("multimat_right_grouped", left, right, 8, n_left=1, n_right=8).astype(np.float64)
+    by_fft = fft.normalize(fft.cross_correlate(left, right, "one_to_many", "original")).astype(np.float64)
+    assert by_fft.shape == by_definition.shape == (8, 511, 511)
+    bound = (2e-5 if dtype == np.float32 else 1e-11) * np.abs(by_definition).max()
+    assert np.abs(by_fft - by_definition).max() <= bound, np.abs(by_fft - by_definition).max() / np.abs(by_definition).max()
