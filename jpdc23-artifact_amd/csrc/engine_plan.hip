@@ -323,9 +323,40 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     return XCORR_OK;
 }
 
+// Planning costs 4-40 microseconds of host time, as much as a small kernel runs: the last few plans are kept per
+// thread and reused when a request differs in its pointers only.
+static bool same_shape(const EngineRequest &a, const EngineRequest &b) {
+    return strcmp(a.family, b.family) == 0 && a.elem_bytes == b.elem_bytes && a.W == b.W && a.H == b.H && a.nV == b.nV && a.nU == b.nU &&
+           a.group_m == b.group_m && a.y_shifts == b.y_shifts && a.x_shifts == b.x_shifts && a.left_mats == b.left_mats &&
+           a.right_mats == b.right_mats && a.lanes_x == b.lanes_x && a.lanes_y == b.lanes_y && a.waves == b.waves &&
+           a.spec_index == b.spec_index && a.rows_per_worker == b.rows_per_worker && a.column_chunks == b.column_chunks &&
+           a.dist == b.dist && a.caller_zeroes == b.caller_zeroes && a.may_split == b.may_split;
+}
+
+static int cached_plan(const EngineRequest &rq, EnginePlan &plan) {
+    struct Entry {
+        bool used;
+        EngineRequest rq;
+        EnginePlan plan;
+    };
+    constexpr int N = 8;
+    thread_local Entry cache[N] = {};
+    thread_local int next = 0;
+    for (int i = 0; i < N; ++i)
+        if (cache[i].used && same_shape(cache[i].rq, rq)) {
+            plan = cache[i].plan;
+            return XCORR_OK;
+        }
+    int rc = plan_engine(rq, plan);
+    if (rc != XCORR_OK) return rc;
+    cache[next] = Entry{true, rq, plan};
+    next = (next + 1) % N;
+    return XCORR_OK;
+}
+
 int run_engine(const EngineRequest &rq, hipStream_t stream) {
     EnginePlan plan;
-    int rc = plan_engine(rq, plan);
+    int rc = cached_plan(rq, plan);
     if (rc != XCORR_OK) return rc;
     rc = rq.elem_bytes == 4 ? launch_typed<float>(rq, plan, stream) : launch_typed<double>(rq, plan, stream);
     if (rc != XCORR_OK) return rc;
