@@ -36,17 +36,17 @@ static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),
     make_spec<R_1x4>("f32_a1b8_r4"),
     make_spec<R_2x2>("f32_a1b8_l2r2"),
-    make_spec<Z_84>("f32_a8b4", 0.755, 0.0),
-    make_spec<Z_88>("f32_a8b8", 0.804, 4.17),
-    make_spec<Z_44>("f32_a4b4", 0.878, 0.0),
-    make_spec<Z_84_u4>("f32_a8b4_lr4", 0.751, 3.75),
-    make_spec<Z_88_u4>("f32_a8b8_lr4", 0.771, 11.78),
-    make_spec<Z_84_u16>("f32_a8b4_lr16", 1.06, 3.399),
-    make_spec<Z_88_u16>("f32_a8b8_lr16", 1.048, 4.906),
-    make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4", 0.861, 0.0),
-    make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.832, 3.941),
-    make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8", 1.078, 0.0),
-    make_spec<Z_84_u8>("f32_a8b4_lr8", 0.773, 7.543),
+    make_spec<Z_84>("f32_a8b4", 0.713, 2.629),
+    make_spec<Z_88>("f32_a8b8", 0.749, 8.237),
+    make_spec<Z_44>("f32_a4b4", 0.833, 0.743),
+    make_spec<Z_84_u4>("f32_a8b4_lr4", 0.66, 5.288),
+    make_spec<Z_88_u4>("f32_a8b8_lr4", 0.692, 10.581),
+    make_spec<Z_84_u16>("f32_a8b4_lr16", 0.9, 4.421),
+    make_spec<Z_88_u16>("f32_a8b8_lr16", 0.875, 8.433),
+    make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4", 0.811, 0.973),
+    make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.727, 6.347),
+    make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8", 0.956, 5.555),
+    make_spec<Z_84_u8>("f32_a8b4_lr8", 0.679, 6.951),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {

@@ -28,16 +28,16 @@ using D_84_v4u8 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 1, 4, 8, 1, 1, 18, 8, 3, 4
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
     make_spec<R_2x2>("f64_a1b4_l2r2"),
-    make_spec<Z_88>("f64_a8b8", 0.706, 0.0),
-    make_spec<Z_44>("f64_a4b4", 0.798, 0.0),
-    make_spec<Z_88_u4>("f64_a8b8_lr4", 0.737, 0.0),
-    make_spec<Z_88_u16>("f64_a8b8_lr16", 0.758, 15.11),
-    make_spec<Z_88_v4u4>("f64_a8b8_ll4lr4", 0.786, 2.096),
-    make_spec<Z_88_v8u8>("f64_a8b8_ll8lr8", 0.726, 20.0),
-    make_spec<Y_84_u4>("f64_a8b4_lr4", 0.735, 0.0),
-    make_spec<Y_84>("f64_a8b4", 0.7, 0.0),
-    make_spec<D_84_v4u4>("f64_a8b4_ll4lr4", 0.767, 0.0),
-    make_spec<D_84_v4u8>("f64_a8b4_ll4lr8", 0.805, 0.0),
+    make_spec<Z_88>("f64_a8b8", 0.705, 0.0),
+    make_spec<Z_44>("f64_a4b4", 0.761, 0.638),
+    make_spec<Z_88_u4>("f64_a8b8_lr4", 0.716, 1.26),
+    make_spec<Z_88_u16>("f64_a8b8_lr16", 0.766, 5.832),
+    make_spec<Z_88_v4u4>("f64_a8b8_ll4lr4", 0.807, 0.137),
+    make_spec<Z_88_v8u8>("f64_a8b8_ll8lr8", 0.637, 12.851),
+    make_spec<Y_84_u4>("f64_a8b4_lr4", 0.733, 0.0),
+    make_spec<Y_84>("f64_a8b4", 0.676, 0.0),
+    make_spec<D_84_v4u4>("f64_a8b4_ll4lr4", 0.768, 0.0),
+    make_spec<D_84_v4u8>("f64_a8b4_ll4lr8", 0.799, 0.0),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {

@@ -138,19 +138,20 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
 //   * a block issues A*B FMAs per lane for every (right row, right column) its shift tile overlaps;
 //     a chunk of rc left rows meets rc + A - 1 right rows, so short chunks pay for the window;
 //   * with many blocks the run is bound by the issue rate of the CUs (average block), with few by
-//     the largest block (the centre tile, all rows and columns) at the issue rate one wavefront per
-//     SIMD reaches alone, which is less than half of what several resident wavefronts reach together;
+//     the largest block (the centre tile, all rows and columns) at the issue rate the few wavefronts
+//     of a SIMD reach together (one alone: 0.6 of what four reach);
 //     the two regimes blend: issue-bound time of all blocks plus a share of the largest block's time;
 //   * every block costs a fixed prologue / epilogue and every staged band a little; a split plan
 //     pays the clear kernel and the atomic adds of all blocks at the rate the memory system takes
 //     them (lower when the lanes of a wavefront write to different result matrices).
 // The constants were fitted to sweeps of all grouped tiles and chunk sizes over 16x16 ... 1024x1024
-// matrices and 1 ... 1024 pairs on MI355X; `issue_factor` and `stage_factor` are per tile.
+// matrices and 1 ... 1024 pairs on MI355X (tuning/sweep_plans.py measures, tuning/fit_planner_model.py fits and
+// mirrors this function); `issue_factor` and `stage_factor` are per tile.
 static double predict_us(const EngineSpec &s, const EngineRequest &rq, const EnginePlan &plan) {
     const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.LV * s.LU > 1;
-    const double t_block = 3.87, e_alone = 0.415, e_full = 0.995, t_stage = 0.0839, k_tail = 0.306;
-    const double t_clear = f32 ? 1.36 : 0.0, t_atomic = f32 ? 0.0384 : 0.0186;
-    const double us_per_atomic = lanes_over_matrices ? (f32 ? 5.4e-6 : 5.1e-6) : (f32 ? 2.9e-6 : 7.2e-6);
+    const double t_block = 4.41, tau = 1.07, e_full = 0.954, t_stage = 0.209, k_tail = 0.281;
+    const double t_clear = f32 ? 1.49 : 0.0, t_atomic = f32 ? 0.0462 : 0.0811;
+    const double us_per_atomic = lanes_over_matrices ? (f32 ? 4.5e-6 : 3.0e-6) : (f32 ? 1.6e-6 : 4.4e-6);
     const double cyc = (f32 ? 2.0 : 4.0) / 2100.0; // microseconds per FMA instruction of a wavefront
     const double W = rq.W, H = rq.H, TXW = s.TXB(), TYW = s.TYB();
     const bool split = plan.atomic != 0;
@@ -172,7 +173,8 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     double n1 = std::ceil(items / cus);
     if (n1 > occ) n1 = occ;
     const double fixed = t_block + (split && !lanes_over_matrices ? t_atomic * s.A * s.B : 0.0);
-    const double crit = fixed + t_stage * stages_max + std::fmax(inst_max * cyc / e_alone, n1 * inst_max * cyc / e_full);
+    // n1 blocks on a CU (one wavefront each per SIMD) issue together at e_full * (1 - exp(-n1 / tau)) of the FMA rate
+    const double crit = fixed + t_stage * stages_max + n1 * inst_max * cyc / (e_full * (1.0 - std::exp(-n1 / tau)));
     const double per_block = (fixed + t_stage * stages_avg) / n1 + inst_avg * cyc / e_full;
     const double tail = k_tail * crit;
     double t = std::fmax(items * per_block / cus + tail, crit);
