@@ -2,7 +2,8 @@
 """Fits the constants of the planner's run-time model (csrc/engine_plan.hip, predict_us) to logs of sweep_plans.py
 and reports how far the model's pick is from the best measured plan of every shape.
 
-  python fit_planner_model.py sweep_f32.log [more logs of the same element type ...] [--fix-global FILE]
+  python fit_planner_model.py sweep_f32.log [more logs of the same element type ...] [--fix-global '...']
+  python fit_planner_model.py sweep_f32.log --installed     # no fit: the constants in the sources against these logs
 
 The model below mirrors predict_us term by term. Fitted by weighted least squares on log(time): plans close
 to the best of their shape weigh most, so that the ranking near the optimum is what the fit gets right.
@@ -88,9 +89,27 @@ def predict(x, names, tiles, r):
     return t
 
 
+def installed_constants(names, f64):
+    """the constants of predict_us and the per-tile factors as they stand in the sources"""
+    text = open(os.path.join(CSRC, "engine_plan.hip")).read()
+    body = text[text.index("static double predict_us"):]
+
+    def pair(name):  # 'name = f32 ? a : b' or 'name = a'
+        m = re.search(name + r" = (?:f32 \? )?([\d.e-]+)(?: : ([\d.e-]+))?", body)
+        return float(m.group(2) if f64 and m.group(2) else m.group(1))
+
+    m = re.search(r"us_per_atomic = lanes_over_matrices \? \(f32 \? ([\d.e-]+) : ([\d.e-]+)\) : \(f32 \? ([\d.e-]+) : ([\d.e-]+)\)", body)
+    lanes, plain = (float(m.group(2)), float(m.group(4))) if f64 else (float(m.group(1)), float(m.group(3)))
+    x = [pair("t_block"), pair("tau"), pair("e_full"), pair("t_stage"), pair("k_tail"), pair("t_clear"), pair("t_atomic"), plain, lanes]
+    tile_text = open(os.path.join(CSRC, "engine_f64.hip" if f64 else "engine_f32.hip")).read()
+    factors = {m.group(1): (float(m.group(2)), float(m.group(3))) for m in re.finditer(r'make_spec<\w+>\("(\w+)", ([\d.]+), ([\d.]+)\)', tile_text)}
+    return x + [factors[n][0] for n in names] + [factors[n][1] for n in names]
+
+
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("logs", nargs="+")
+    ap.add_argument("--installed", action="store_true", help="do not fit: evaluate the constants that stand in the sources")
     ap.add_argument("--fix-global", default=None, metavar="'t_block tau e_full t_stage k_tail'")
     a = ap.parse_args()
     tiles = tile_table()
@@ -109,9 +128,13 @@ def main():
     def residuals(x):
         return [math.log(predict(x, names, tiles, r) / r["us"]) * (best[r["shape"]] / r["us"]) ** 1.5 for r in rows]
 
-    sol = least_squares(residuals, x0, bounds=(lo, hi))
-    x = sol.x
-    print(f"{len(rows)} measurements, weighted rms of log(model / measured) = {np.sqrt(np.mean(np.square(sol.fun))):.3f}")
+    if a.installed:
+        x = np.array(installed_constants(names, rows[0]["f64"]))
+        print(f"{len(rows)} measurements, constants of the sources, weighted rms of log(model / measured) = {np.sqrt(np.mean(np.square(residuals(x)))):.3f}")
+    else:
+        sol = least_squares(residuals, x0, bounds=(lo, hi))
+        x = sol.x
+        print(f"{len(rows)} measurements, weighted rms of log(model / measured) = {np.sqrt(np.mean(np.square(sol.fun))):.3f}")
     print("t_block tau e_full t_stage k_tail =", " ".join(f"{v:.4g}" for v in x[:5]))
     print("t_clear t_atomic us_per_atomic(plain) us_per_atomic(lanes over matrices) =", " ".join(f"{v:.4g}" for v in x[5:9]))
     for i, n in enumerate(names):

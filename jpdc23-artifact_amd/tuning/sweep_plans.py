@@ -57,7 +57,8 @@ def main():
         label = f"{shape}:{a.dtype}"
 
         def measure(spec, rows):
-            params = xc.make_params(specialisation=spec, rows_per_thread=rows)
+            # forced plans are not cut over columns (the model covers row chunks only); the planner's pick may be
+            params = xc.make_params(specialisation=spec, rows_per_thread=rows, column_chunks=1 if spec else 0)
 
             def go():
                 xc.launch(FAMILY[mode], d_left, d_right, d_out, size, size, n_left, per_left, dtype, params)
