@@ -449,15 +449,17 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     xr_lo = (xr_lo / C::KBX) * C::KBX;
     int xr_hi = W - sxb;
     if (xr_hi > W) xr_hi = W;
-    // this work item's chunk of those columns
-    int col_lo = 0, col_hi = W;
+    // this work item's chunk of those columns: [xr_lo, xr_hi) shrinks to it, and w_hi (= W when the
+    // columns are not cut) bounds the columns a partial last stage may sweep
+    int w_hi = W;
     if (g.x_chunks > 1) {
-        col_lo = xr_lo + xch * g.x_chunk_cols;
-        col_hi = col_lo + g.x_chunk_cols;
-        if (col_hi > xr_hi) col_hi = xr_hi;
-        if (col_lo >= col_hi) return; // the tile overlaps fewer columns than the widest one
-        xr_lo = (col_lo / C::KBX) * C::KBX;
-        xr_hi = col_hi;
+        const int lo = xr_lo + xch * g.x_chunk_cols;
+        int hi = lo + g.x_chunk_cols;
+        if (hi > xr_hi) hi = xr_hi;
+        if (lo >= hi) return; // the tile overlaps fewer columns than the widest one
+        xr_lo = lo;
+        xr_hi = hi;
+        w_hi = hi;
     }
 
     // ---- lane coordinates ----
@@ -544,14 +546,9 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             int need = -(sxw + C::TXW - 1) - (K - 1) - x0;
             if (need > 0) kc_lo = (need + K - 1) / K;
             int lim = W - 1 - sxw - x0;
-            if (W - 1 - x0 < lim) lim = W - 1 - x0;
+            if (w_hi - 1 - x0 < lim) lim = w_hi - 1 - x0;
             int h = lim < 0 ? 0 : lim / K + 1;
             if (h < kc_hi) kc_hi = h;
-        }
-        if (g.x_chunks > 1) {
-            const int lo = (col_lo - x0) / K, hi = (col_hi - x0 + K - 1) / K; // col_lo - x0 is a multiple of K or negative
-            if (col_lo > x0 && lo > kc_lo) kc_lo = lo;
-            if (hi < kc_hi) kc_hi = hi;
         }
         if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
         if (jj_lo < jj_hi || (jj_lo == jj_hi && tail > 0))

@@ -30,7 +30,8 @@ using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 18, 16, 4, 4
 using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 18, 16, 4, 4>;
-using Z_84_u8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 4, 4>;
+// (168 registers, three wavefronts per SIMD: the eight band offsets per lane spill less, measured 1.6 % faster than at 128)
+using Z_84_u8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 3, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),
@@ -46,7 +47,7 @@ static const EngineSpec specs[] = {
     make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4", 0.811, 0.973),
     make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.727, 6.347),
     make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8", 0.956, 5.555),
-    make_spec<Z_84_u8>("f32_a8b4_lr8", 0.679, 6.951),
+    make_spec<Z_84_u8>("f32_a8b4_lr8", 0.64, 6.951),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {
