@@ -289,6 +289,20 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
             if (rc <= 0) rc = rq.H;
         }
     }
+    if (rq.caller_zeroes && rc <= 0 && rq.dist != XCORR_DIST_NONE) {
+        // split-row contract without a chunk size from the caller: the longest chunk of 8, 4, 2 staged bands that
+        // still gives every CU eight work items, else one band (n-to-m 16 x 32 of 64x64 fp64: 1.30 -> 0.76 ms
+        // against one band; a single pair of small matrices keeps the short chunks it needs to fill the GPU)
+        rc = best->RL;
+        for (int k = 8; k > 1; k /= 2) {
+            EnginePlan longer;
+            if (int e = shape_plan(*best, rq, k * best->RL, 1, longer)) return e;
+            if (longer.total_items >= 8L * device_cus()) {
+                rc = k * best->RL;
+                break;
+            }
+        }
+    }
     return shape_plan(*best, rq, rc, 1, plan);
 }
 
