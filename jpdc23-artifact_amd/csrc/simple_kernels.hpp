@@ -99,6 +99,7 @@ int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsig
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if (n_left == 0 || batch == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if (batch > 0x7fffffffu) return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: batch of %u", batch);
     const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
     dim3 block(64, 4);
     unsigned long long strip = (unsigned long long)Sx * n_left;

@@ -276,7 +276,7 @@ int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, un
     const xcorr_params &p = params_or_default(pp);
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
-    if (n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no right matrices");
+    if ((rc = check_counts(1, n_right, false))) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
@@ -300,7 +300,7 @@ int multimat_right_grouped_impl(const T *left, const T *right, T *out, unsigned 
     const xcorr_params &p = params_or_default(pp);
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
-    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_counts(n_left, n_right, true))) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("shifts per thread per right matrix", p.shifts_per_thread_right_matrix, Limits::combined))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::combined))) return rc;
@@ -324,7 +324,7 @@ int multimat_both_impl(const T *left, const T *right, T *out, unsigned cols, uns
     const xcorr_params &p = params_or_default(pp);
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
-    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_counts(n_left, n_right, true))) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("left matrices per thread", p.left_matrices_per_thread, Limits::left_matrices))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
@@ -345,7 +345,7 @@ int multimat_both_grouped_impl(const T *left, const T *right, T *out, unsigned c
     const xcorr_params &p = params_or_default(pp);
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
-    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    if ((rc = check_counts(n_left, n_right, true))) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("shifts per thread per right matrix", p.shifts_per_thread_right_matrix, Limits::combined))) return rc;
     if ((rc = check_limit("left matrices per thread", p.left_matrices_per_thread, Limits::combined))) return rc;

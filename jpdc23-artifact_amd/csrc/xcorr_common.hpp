@@ -72,4 +72,13 @@ inline int check_shape(const void *left, const void *right, const void *out, uns
     return XCORR_OK;
 }
 
+// matrix counts and the number of result matrices are 32-bit signed in the planner and the kernels
+inline int check_counts(unsigned n_left, unsigned n_right, bool all_pairs) {
+    if (n_left == 0 || n_right == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
+    const unsigned long long results = all_pairs ? (unsigned long long)n_left * n_right : n_right;
+    if (n_left > 0x7fffffffu || n_right > 0x7fffffffu || results > 0x7fffffffull)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: %u left, %u right", n_left, n_right);
+    return XCORR_OK;
+}
+
 } // namespace xcorr

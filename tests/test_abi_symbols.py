@@ -73,6 +73,15 @@ def test_argument_errors_without_a_device():
     p = xc.make_params(block_size=2048)
     assert lib.xcorr_block_per_overlap_f32(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None) == 1
     assert b"Thread block too large: 2048 (max 1024)" in lib.xcorr_last_error()
+    # matrix counts whose product leaves the 31-bit range of the work-item arithmetic
+    assert lib.xcorr_multimat_both_grouped_f32(dummy, dummy, dummy, 8, 8, 1 << 16, 1 << 16, None, None) == 1
+    assert b"too many matrices: 65536 left, 65536 right" in lib.xcorr_last_error()
+    assert lib.xcorr_multimat_right_grouped_f64(dummy, dummy, dummy, 8, 8, 3, 0xC0000000, None, None) == 1
+    assert b"too many matrices" in lib.xcorr_last_error()
+    assert lib.xcorr_multimat_right_f32(dummy, dummy, dummy, 8, 8, 0, None, None) == 1
+    assert b"no matrices" in lib.xcorr_last_error()
+    assert lib.xcorr_overlap_wise_f32(dummy, dummy, dummy, 8, 8, 1, 0x80000000, None) == 1
+    assert b"too many matrices" in lib.xcorr_last_error()
     rec = xc.LaunchRecord()
     assert lib.xcorr_last_launch(ctypes.byref(rec)) == 1
     assert b"No kernel launch" in lib.xcorr_last_error()
