@@ -39,12 +39,17 @@ struct EngineSpec {
 
 template <class C>
 hipError_t allow_large_lds() {
-    static bool attr_set = false;
-    if (!attr_set && C::LDS_BYTES > 64 * 1024) {
+    if (C::LDS_BYTES <= 64 * 1024) return hipSuccess;
+    // the attribute belongs to the kernel's copy on one device: kept per device of the process
+    static bool attr_set[64] = {};
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+    const bool tracked = dev >= 0 && dev < 64;
+    if (!tracked || !attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&engine_kernel<C>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return e;
-        attr_set = true;
+        if (tracked) attr_set[dev] = true;
     }
     return hipSuccess;
 }
