@@ -77,6 +77,10 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch the library's plain copy kernel on 256 MiB so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
                          "readings of the same run can be scaled to bytes")
+    ap.add_argument("--data", choices=["config", "integers", "zeros"], default="config",
+                    help="input values: the configuration's seeded distribution (default; what the figures are quoted on), "
+                         "small integers, or zeros. The kernels execute the same instructions for any values, but the shader "
+                         "clock of the GPU is power-managed and runs 10-15 %% higher when few operand bits toggle")
     ap.add_argument("--graph-replay", type=int, default=0, metavar="N",
                     help="additionally capture N steps into one HIP graph and time its replays (reported under \"graph_replay\")")
     args = ap.parse_args()
@@ -91,7 +95,9 @@ def main():
     cfg = dict(workloads.CONFIGS[args.config], name=args.config)
     family = args.family or cfg["family"]
     dtype = np.dtype(cfg["dtype"])
-    left, right = workloads.generate(cfg)
+    left, right = workloads.generate(cfg, integer_valued=args.data != "config")
+    if args.data == "zeros":
+        left, right = np.zeros_like(left), np.zeros_like(right)
     rows, cols = cfg["rows"], cfg["cols"]
     pairs = workloads.num_pairs(cfg)
     n_left = cfg["n_left"]
@@ -205,7 +211,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32" if dtype == np.float32 else "f64",
-        "data": "synthetic",
+        "data": "synthetic" if args.data == "config" else f"synthetic ({args.data})",
         "config": {
             "workload": f"{args.config}: {cfg['mode']} {cfg['n_left']}x{cfg['n_right']} matrices of {rows}x{cols} {cfg['dtype']}, "
                         f"{cfg['dist']} seed {cfg['seed']}, family {family}",
@@ -225,7 +231,8 @@ def main():
             "algorithmic_bytes": workloads.algorithmic_bytes(cfg),
             "kernel_ms": round(kernel_ms, 4),
             "note": "vector-FMA roofline (MFMA is not used); the kernel issues plain v_fmac_f32, which measures "
-                    "0.97 of this peak in a register-only loop on MI355X" if dtype == np.float32 else
+                    "0.97 of this peak in a register-only loop on MI355X; the peak assumes 2.4 GHz, the power-managed "
+                    "shader clock under this kernel is 2.0-2.1 GHz on random data (2.37 GHz with --data integers)" if dtype == np.float32 else
                     "vector-FMA roofline, v_fma_f64",
         },
     }
