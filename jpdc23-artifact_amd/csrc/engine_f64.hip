@@ -25,6 +25,10 @@ using Y_84 = EngineCfg<double, 8, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 3, 4>;
 using D_84_v4u4 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 2, 4, 4, 1, 1, 18, 8, 3, 4, 1>;
 using D_84_v4u8 = EngineCfg<double, 8, 4, 2, 1, 1, 2, 1, 4, 8, 1, 1, 18, 8, 3, 4, 1>;
 
+// 4x4 tiles with lanes over right matrices, for many small matrices
+using Z_44_u4 = EngineCfg<double, 4, 4, 2, 1, 1, 4, 4, 1, 4, 1, 1, 20, 8, 4, 4>;
+using Z_44_u8 = EngineCfg<double, 4, 4, 2, 1, 1, 4, 2, 1, 8, 1, 1, 20, 8, 4, 4>;
+
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f64_a1b8"),
     make_spec<R_2x2>("f64_a1b4_l2r2"),
@@ -38,6 +42,8 @@ static const EngineSpec specs[] = {
     make_spec<Y_84>("f64_a8b4", 0.676, 0.0),
     make_spec<D_84_v4u4>("f64_a8b4_ll4lr4", 0.768, 0.0),
     make_spec<D_84_v4u8>("f64_a8b4_ll4lr8", 0.799, 0.0),
+    make_spec<Z_44_u4>("f64_a4b4_lr4", 0.82, 1.0),
+    make_spec<Z_44_u8>("f64_a4b4_lr8", 0.85, 1.0),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {

@@ -330,7 +330,7 @@ def test_reduction_cut_over_columns(oracle, dtype):
     instead of, the cut over left rows); every grouped tile, more chunks than columns allow, ragged widths."""
     xc = load_package()
     rng = np.random.default_rng(900)
-    n_specs = 15 if dtype == np.float32 else 12
+    n_specs = 17 if dtype == np.float32 else 14
     first_grouped = 4 if dtype == np.float32 else 3
     for family, mode, n_left, n_right, shape in [("grouped_overlap", "one_to_one", 1, 1, (40, 70)),
                                                  ("multimat_right_grouped", "one_to_many", 1, 5, (33, 18)),
