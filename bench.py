@@ -24,7 +24,7 @@ PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
 # by the library's copy kernel (figures and commands: profiles/engine_f32_a8b4_one_to_one_1024.md, profiles/engine_other_workloads.md).
 # Measured for the default parameters of each workload only (fetched + written).
-MEASURED_TRAFFIC_BYTES = {"C2": 2.232e9 + 0.636e9, "C3": 0.218e9 + 0.231e9, "C4": 0.279e9 + 0.193e9, "C5": 0.006e9 + 0.108e9}
+MEASURED_TRAFFIC_BYTES = {"C2": 2.232e9 + 0.636e9, "C3": 0.0253e9 + 0.143e9, "C4": 0.0114e9 + 0.062e9, "C5": 0.006e9 + 0.108e9}
 
 
 def cpu_baseline(oracle, cfg, left, right, budget_s=15.0):
