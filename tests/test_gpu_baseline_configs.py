@@ -211,3 +211,27 @@ def test_output_larger_than_2_32_elements(oracle):
         centre = fetch(pair)[size - 1, size - 1]
         assert centre == float(np.sum(left[l].astype(np.float64) * right[r])), pair
     d_out.free()
+
+
+@pytest.mark.parametrize("rows,cols,dtype,family", [(3000, 2500, np.float32, "grouped_overlap"),
+                                                    (1537, 4099, np.float64, "grouped_overlap"),
+                                                    (2049, 1023, np.float32, "split_row"),
+                                                    (700, 9000, np.float32, "grouped_overlap")])
+def test_large_non_square_pair_spot_checked(rows, cols, dtype, family):
+    """Single pairs beyond the benchmark sizes (up to 7.5e6 elements per matrix, ragged against every tile and
+    staging width): too large for the oracle's loop, so the corners, the centre and 300 random result elements
+    are compared with the definition evaluated for that element alone (values in {-1, 0, 1}: every sum is exact)."""
+    xc = load_package()
+    rng = np.random.default_rng(5)
+    left = rng.integers(-1, 2, (rows, cols)).astype(dtype)
+    right = rng.integers(-1, 2, (rows, cols)).astype(dtype)
+    print("case", family, rows, cols, np.dtype(dtype).name, flush=True)
+    got = xc.run(family, left, right, 1)[0]
+    points = [(0, 0), (2 * rows - 2, 2 * cols - 2), (rows - 1, cols - 1), (0, 2 * cols - 2), (2 * rows - 2, 0)]
+    points += [(int(rng.integers(0, 2 * rows - 1)), int(rng.integers(0, 2 * cols - 1))) for _ in range(300)]
+    for oy, ox in points:
+        sy, sx = oy - (rows - 1), ox - (cols - 1)
+        y0, y1 = max(0, -sy), min(rows, rows - sy)
+        x0, x1 = max(0, -sx), min(cols, cols - sx)
+        exp = float(np.sum(left[y0 + sy:y1 + sy, x0 + sx:x1 + sx].astype(np.float64) * right[y0:y1, x0:x1].astype(np.float64)))
+        assert got[oy, ox] == exp, (oy, ox, got[oy, ox], exp, xc.last_launch()["kernel"])
