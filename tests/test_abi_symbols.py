@@ -73,6 +73,8 @@ def test_argument_errors_without_a_device():
     p = xc.make_params(block_size=2048)
     assert lib.xcorr_block_per_overlap_f32(dummy, dummy, dummy, 8, 8, ctypes.byref(p), None) == 1
     assert b"Thread block too large: 2048 (max 1024)" in lib.xcorr_last_error()
+    assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 16385, 8, None, None) == 1
+    assert b"matrix too large: 8 x 16385 (max 16384)" in lib.xcorr_last_error()
     # matrix counts whose product leaves the 31-bit range of the work-item arithmetic
     assert lib.xcorr_multimat_both_grouped_f32(dummy, dummy, dummy, 8, 8, 1 << 16, 1 << 16, None, None) == 1
     assert b"too many matrices: 65536 left, 65536 right" in lib.xcorr_last_error()
