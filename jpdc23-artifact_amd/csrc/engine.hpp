@@ -114,48 +114,6 @@ struct vec128<double> {
     typedef double type __attribute__((ext_vector_type(2)));
 };
 
-// Cycle accounting per phase of engine_kernel, compiled in with -DXCORR_ENGINE_PROFILE only (a
-// tuning aid: every wavefront adds the shader-clock cycles it spent per phase to a device-side
-// table that engine_profile_read() copies out and clears).
-enum EnginePhase { PH_SETUP, PH_WAIT_SIBLINGS, PH_STAGING, PH_WAIT_STAGED, PH_COMPUTE, PH_OUTPUT, PH_DECODE, PH_COUNT };
-#ifdef XCORR_ENGINE_PROFILE
-static __device__ unsigned long long engine_profile[PH_COUNT + 3]; // phases, wavefronts, first-to-last cycles, same in 100 MHz ticks
-struct PhaseClock {
-    long long t0, t, w0, acc[PH_COUNT];
-    __device__ __forceinline__ PhaseClock() {
-        for (int i = 0; i < PH_COUNT; ++i) acc[i] = 0;
-        t0 = t = (long long)clock64();
-        w0 = (long long)wall_clock64();
-    }
-    __device__ __forceinline__ void lap(int phase) {
-        long long now = (long long)clock64();
-#pragma unroll
-        for (int i = 0; i < PH_COUNT; ++i) // (no dynamic indexing: the table stays in registers)
-            if (i == phase) acc[i] += now - t;
-        t = now;
-    }
-    __device__ __forceinline__ void flush() {
-        if ((threadIdx.x & 63) == 0) {
-            for (int i = 0; i < PH_COUNT; ++i) atomicAdd(&engine_profile[i], (unsigned long long)acc[i]);
-            atomicAdd(&engine_profile[PH_COUNT], 1ull);
-            atomicAdd(&engine_profile[PH_COUNT + 1], (unsigned long long)(t - t0));
-            atomicAdd(&engine_profile[PH_COUNT + 2], (unsigned long long)((long long)wall_clock64() - w0));
-        }
-    }
-};
-static inline hipError_t engine_profile_read(unsigned long long *out) {
-    hipError_t e = hipMemcpyFromSymbol(out, HIP_SYMBOL(engine_profile), sizeof(engine_profile));
-    if (e != hipSuccess) return e;
-    unsigned long long zero[PH_COUNT + 3] = {};
-    return hipMemcpyToSymbol(HIP_SYMBOL(engine_profile), zero, sizeof(zero));
-}
-#else
-struct PhaseClock {
-    __device__ __forceinline__ void lap(int) {}
-    __device__ __forceinline__ void flush() {}
-};
-#endif
-
 __device__ __forceinline__ void atomic_add(float *p, float v) { unsafeAtomicAdd(p, v); }
 __device__ __forceinline__ void atomic_add(double *p, double v) { unsafeAtomicAdd(p, v); }
 
@@ -214,19 +172,17 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
     }
 }
 
-// Lane i of the wavefront copies the 16 bytes at its own global address to LDS byte address
-// lds_base + 16 * i, without passing through registers; completion is counted by vmcnt. The
-// compiler does not know that this writes LDS: callers wait (dma_wait) and pass a barrier before
-// anything reads the destination.
-// (M0, which carries the LDS address, is a register the compiler reserves for uses of this
-// kind and never keeps a value in across statements; naming it as clobbered states the fact and
-// draws a warning about reserved registers, silenced here.)
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void dma16(const void *gptr, unsigned lds_base) {
-    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_base) : "memory", "m0");
+// Lane i of the wavefront copies the 16 bytes at its own global address to LDS address
+// lds_wave_base + 16 * i, without passing through registers; completion is counted by vmcnt.
+// `lds_wave_base` must be the same for all lanes. The LDS address travels in M0; the compiler
+// builtin is used (not inline assembly) so that the compiler writes M0 itself and keeps the wait
+// state the hardware needs between an SALU write of M0 and the LDS-DMA instruction that reads it.
+// The compiler does not order ordinary LDS reads after this copy: callers wait (dma_wait) and
+// pass a barrier before anything reads the destination.
+__device__ __forceinline__ void dma16(const void *gptr, void *lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr,
+                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
-#pragma clang diagnostic pop
 __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // stage_bands with the copies done by dma16: pieces that lie fully inside the matrices are copied
@@ -243,9 +199,8 @@ __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, c
     constexpr int VK = C::VK, PP = PITCH / VK, BANDP = BAND / VK, TOTP = NB * BANDP;
     constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
     static_assert(PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
-    // LDS byte address of the piece of lane 0 of this wavefront in iteration 0
-    const unsigned wave_base =
-        __builtin_amdgcn_readfirstlane((unsigned)(size_t)lds) + (unsigned)__builtin_amdgcn_readfirstlane(tid & ~63) * 16u;
+    // first 128-bit piece of this wavefront in iteration 0 (the same for all its lanes)
+    const int wave_piece = __builtin_amdgcn_readfirstlane(tid & ~63);
 #pragma unroll
     for (int it = 0; it < ITER; ++it) {
         const int p = tid + it * C::NT;
@@ -254,7 +209,7 @@ __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, c
             const bool inside = band < nbands && row >= row_lo && row < row_hi;
             const T *gp = src + (size_t)band * mat_stride + (ptrdiff_t)(row0 + row) * W + (ptrdiff_t)(col0 + col);
             if (inside && col >= col_lo && col + VK <= col_hi) {
-                dma16(gp, wave_base + (unsigned)(it * C::NT) * 16u);
+                dma16(gp, lds + (size_t)(wave_piece + it * C::NT) * VK);
             } else {
                 // zero the piece, then patch in the elements of a piece that straddles an edge (the
                 // patch is kept apart from the zeroing so that only it waits for its loads)
@@ -383,7 +338,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     T *Us = Vs + C::NVB * C::VBAND;
     const int W = g.W, H = g.H;
 
-    PhaseClock pc;
     // ---- decode the work item (uniform over the threads that share it) ----
     int item = (int)blockIdx.x;
     if (item >= g.total_items) return;
@@ -428,7 +382,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     if (chi > row_hi) chi = row_hi;
     if (clo >= chi) return; // surplus worker of the rectangle distribution
 
-    pc.lap(PH_DECODE);
     const int syb = -(H - 1) + ty * C::TYB;
     const int sxb = -(W - 1) + tx * C::TXB;
 
@@ -560,10 +513,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         if (nstages > 0) stage(Vs, clo, xr_lo);
         int yl0 = clo, x0 = xr_lo; // stage being computed
         for (int st = 0; st < nstages; ++st) {
-            pc.lap(st == 0 ? PH_SETUP : PH_COMPUTE);
             dma_wait();
             __syncthreads(); // stage st has landed for everyone, and everyone is done with stage st-1
-            pc.lap(PH_WAIT_STAGED);
             int yl1 = yl0, x1 = x0 + C::KBX;
             if (x1 >= xr_hi) {
                 x1 = xr_lo;
@@ -571,29 +522,21 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             }
             const int cur = (st & 1) * C::LDS_ELEMS;
             if (st + 1 < nstages) stage(Vs + (C::LDS_ELEMS - cur), yl1, x1);
-            pc.lap(PH_STAGING);
             compute(cur, yl0, x0);
             yl0 = yl1;
             x0 = x1;
         }
     } else {
-        bool first_stage = true;
         for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
             for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
-                pc.lap(first_stage ? PH_SETUP : PH_COMPUTE);
-                first_stage = false;
                 __syncthreads(); // everyone is done reading the previous stage
-                pc.lap(PH_WAIT_SIBLINGS);
                 stage(Vs, yl0, x0);
-                pc.lap(PH_STAGING);
                 __syncthreads();
-                pc.lap(PH_WAIT_STAGED);
                 compute(0, yl0, x0);
             }
         }
     }
 
-    pc.lap(PH_COMPUTE);
     // ---- write the register tiles ----
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     const size_t out_area = (size_t)Sx * Sy;
@@ -667,8 +610,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                 }
             }
         }
-        pc.lap(PH_OUTPUT);
-        pc.flush();
         return;
     }
 #pragma unroll
@@ -698,8 +639,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             }
         }
     }
-    pc.lap(PH_OUTPUT);
-    pc.flush();
 }
 
 // fills n elements with zero (a plain kernel rather than a memset node, so callers may capture it)

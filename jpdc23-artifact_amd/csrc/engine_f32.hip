@@ -69,8 +69,3 @@ const EngineSpec *engine_specs_f32(int *count) {
 }
 
 } // namespace xcorr
-
-#ifdef XCORR_ENGINE_PROFILE
-// profile builds only: copies out and clears the per-phase cycle table of the f32 kernels
-extern "C" int xcorr_debug_engine_profile_f32(unsigned long long *out) { return (int)xcorr::engine_profile_read(out); }
-#endif

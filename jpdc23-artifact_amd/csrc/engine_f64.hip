@@ -52,8 +52,3 @@ const EngineSpec *engine_specs_f64(int *count) {
 }
 
 } // namespace xcorr
-
-#ifdef XCORR_ENGINE_PROFILE
-// profile builds only: copies out and clears the per-phase cycle table of the f64 kernels
-extern "C" int xcorr_debug_engine_profile_f64(unsigned long long *out) { return (int)xcorr::engine_profile_read(out); }
-#endif

@@ -145,8 +145,8 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
 //     pays the clear kernel and the atomic adds of all blocks at the rate the memory system takes
 //     them (lower when the lanes of a wavefront write to different result matrices).
 // The constants were fitted to sweeps of all grouped tiles and chunk sizes over 16x16 ... 1024x1024
-// matrices and 1 ... 1024 pairs on MI355X (tuning/sweep_plans.py measures, tuning/fit_planner_model.py fits and
-// mirrors this function); `issue_factor` and `stage_factor` are per tile.
+// matrices and 1 ... 1024 pairs on MI355X (weighted least squares on the logarithm of the run time);
+// `issue_factor` and `stage_factor` are per tile.
 static double predict_us(const EngineSpec &s, const EngineRequest &rq, const EnginePlan &plan) {
     const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.LV * s.LU > 1;
     const double t_block = 4.41, tau = 1.07, e_full = 0.954, t_stage = 0.209, k_tail = 0.281;

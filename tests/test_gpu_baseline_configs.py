@@ -1,7 +1,9 @@
 """The five benchmark configurations at their full sizes, through the C ABI.
 
-The CPU oracle needs minutes to hours at these sizes, so parity is established through
-properties that do not depend on size:
+C1, C4 and C5 completely, and four of the 64 right matrices of C3, are compared with the CPU
+oracle itself on the seeded inputs (a few seconds of its loop on 16 threads each); C2 on a band of
+central output rows. Besides that, parity is established through properties that do not
+depend on size:
   * integer-valued inputs: every product and partial sum is an exactly representable integer,
     so the result is independent of the summation order and must equal, bit for bit, the
     correlation computed with double-precision FFTs and rounded to the nearest integer (the FFT
@@ -104,6 +106,43 @@ def test_seeded_inputs_within_tolerance_at_full_size(name, family):
     assert err <= tol
 
 
+def oracle_full(oracle, cfg, left, right, threads=16):
+    """The oracle's mode driver for a configuration (inputs and results in file order)."""
+    fn = {"one_to_one": oracle.one_to_one, "one_to_many": oracle.one_to_many, "n_to_mn": oracle.n_to_mn, "n_to_m": oracle.n_to_m}[cfg["mode"]]
+    return fn(left if cfg["mode"] not in ("one_to_one", "one_to_many") else left[0], right if cfg["mode"] != "one_to_one" else right[0],
+              threads=threads)
+
+
+@pytest.mark.parametrize("name,subset", [("C1", None), ("C3", 4), ("C4", None), ("C5", None)])
+def test_seeded_inputs_against_the_oracle_at_full_size(oracle, name, subset):
+    """The default launch of a configuration against the oracle's own loop on the same seeded inputs
+    (the reference's host result, validate.hpp:94-132 and its mode drivers :216-298): relative Frobenius
+    error at most 1e-5 (fp32) / 1e-12 (fp64) over ALL results, max element error printed. C3 costs the
+    oracle 2.7e11 FMAs, so the GPU runs all 64 right matrices and four of them (first, two in the
+    middle, last) are compared."""
+    xc = load_package()
+    from jpdc23_artifact_amd import workloads
+
+    cfg = dict(workloads.CONFIGS[name])
+    left, right = workloads.generate(cfg)
+    print(name, cfg["mode"], left.shape, right.shape, flush=True)
+    got = run_config(xc, cfg, left, right)
+    kernel = xc.last_launch()["kernel"]
+    if subset:
+        picks = sorted({0, cfg["n_right"] // 3, (2 * cfg["n_right"]) // 3, cfg["n_right"] - 1})[:subset]
+        exp = oracle.one_to_many(left[0], right[picks], threads=16)
+        got = got[picks]
+    else:
+        exp = oracle_full(oracle, cfg, left, right)
+    assert got.shape == exp.shape
+    e = oracle.errors(got, exp)
+    tol = 1e-5 if cfg["dtype"] == "float32" else 1e-12
+    print(f"{name} {kernel} vs oracle: rel_frobenius={e.rel_frobenius:.3e} max_abs={e.max_abs:.3e} max_rel={e.max_rel:.3e} "
+          f"max|ref|={np.abs(exp).max():.3e} ({exp.shape[0]} results)", flush=True)
+    assert np.isfinite(got).all()
+    assert e.rel_frobenius <= tol
+
+
 def test_all_ones_closed_form_1024():
     xc = load_package()
     n = 1024
@@ -128,6 +167,9 @@ def test_c2_band_against_oracle(oracle):
       * the one-accumulator-per-output-element family (`shuffle`: every accumulator runs over the
         whole overlap like a thread of the reference's kernel does) reproduces the fp32 host loop
         itself to 1e-5.
+    The default launch therefore MISSES the 1e-5 bar against the fp32 host loop on this configuration
+    (about 1.0e-4); what is asserted about that distance is that it is explained by the host loop's own
+    rounding: no larger than the loop's distance from the exact sum plus 1e-5.
     All pairwise differences are printed with their max element error."""
     xc = load_package()
     from jpdc23_artifact_amd import workloads
@@ -148,6 +190,7 @@ def test_c2_band_against_oracle(oracle):
           f"rel_frobenius={e32.rel_frobenius:.3e} max_abs={e32.max_abs:.3e} max_rel={e32.max_rel:.3e}", flush=True)
     print(f"default vs fp64-accumulated: rel_frobenius={e64.rel_frobenius:.3e} max_abs={e64.max_abs:.3e}", flush=True)
     assert e64.rel_frobenius <= 1e-5
+    assert e32.rel_frobenius <= o64.rel_frobenius + 1e-5
 
     got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(rows_per_thread=1024))[0]
     rec = xc.last_launch()
