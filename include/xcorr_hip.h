@@ -89,7 +89,9 @@ typedef struct xcorr_params {
     unsigned block_size;                     /* block-per-overlap: threads per block, 0 = 128, <= 1024 */
     unsigned column_chunks;                  /* grouped families: cut the reduction over right columns into this many chunks
                                                 (atomic adds, like rows_per_thread for rows); 0 = planner decides, no counterpart in the reference */
-    unsigned reserved;
+    unsigned whole_pair_in_lds;              /* grouped-overlap, one small pair: 0 = the launcher decides, 1 = always run the kernel that
+                                                keeps both matrices in LDS (an error if they do not fit), 2 = never; no counterpart
+                                                in the reference */
 } xcorr_params;
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the
@@ -228,7 +230,12 @@ int xcorr_split_row_f64(const double *left, const double *right, double *out, un
 /* Grouped-overlap: every lane accumulates p->shifts_per_thread adjacent y shifts.
  * Replaces run_ccn_shuffle_multirow_both (kernels.cuh:185-195). One pair.
  * `out` need not be zeroed: when the launcher splits the reduction to fill the
- * device it clears `out` itself on `stream` first. */
+ * device it clears `out` itself on `stream` first. A pair small enough for both
+ * matrices to sit in the LDS of one CU (up to about 128 x 128 fp32) and given no tile
+ * selection runs a kernel of its own kind instead: every block keeps the whole pair
+ * in LDS and its wavefronts reduce groups of four adjacent x shifts, one launch,
+ * no atomics (the role of run_ccn_warp_per_shift_shared_mem, kernels.cuh:144-161, at
+ * such sizes); p->whole_pair_in_lds forces or forbids it. */
 int xcorr_grouped_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                               const xcorr_params *p, void *stream);
 int xcorr_grouped_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,

@@ -51,7 +51,7 @@ class Params(ctypes.Structure):
         ("column_group_per_block", ctypes.c_uint),
         ("block_size", ctypes.c_uint),
         ("column_chunks", ctypes.c_uint),
-        ("reserved", ctypes.c_uint),
+        ("whole_pair_in_lds", ctypes.c_uint),
     ]
 
 

@@ -228,7 +228,9 @@ __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, c
 }
 
 // Inner loops of one stage for one lane: for every K-column chunk kc in [kc_lo, kc_hi) sweep
-// the groups of G staged left rows jj in [jj_lo, jj_hi) and `tail` (< G) more rows after them.
+// the staged left rows from `row0` on: `groups` groups of G rows and `tail` (< G) more rows after
+// them. (The sweep starts at the first row that can overlap this wavefront's shifts, not at a
+// multiple of G: on small matrices the rows before it were a tenth of the work.)
 //
 // Register plan per lane: NV*NU*A*B accumulators, a ring of G = A+1 right rows (row j in
 // slot j mod G, so the row of the next step is fetched while the current step still uses
@@ -241,14 +243,14 @@ __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, c
 template <class C>
 __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
                                               typename C::value_type (&acc)[C::NV][C::NU][C::A][C::B], int kc_lo,
-                                              int kc_hi, int jj_lo, int jj_hi, int tail) {
+                                              int kc_hi, int row0, int groups, int tail) {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     constexpr int A = C::A, B = C::B, K = C::K, NV = C::NV, NU = C::NU, VK = C::VK, G = C::G;
     constexpr int VW = C::VWIN_VECS * VK;
     for (int kc = kc_lo; kc < kc_hi; kc += C::WZ) { // (kc_lo is this wavefront's first chunk)
-        const T *vp = Vs_lane + kc * K + jj_lo * G * C::PV;
-        const T *up = Us_lane + kc * K + jj_lo * G * C::PU;
+        const T *vp = Vs_lane + kc * K + row0 * C::PV;
+        const T *up = Us_lane + kc * K + row0 * C::PU;
         T ring[NU][G][K];
         T vw[NV][VW];
         // rows -(A-1) .. 0 of the right band, window of left row 0
@@ -317,7 +319,7 @@ __device__ __forceinline__ void compute_stage(const typename C::value_type *Vs_l
             }
         };
 #pragma unroll 1
-        for (int jj = jj_lo; jj < jj_hi; ++jj) {
+        for (int jj = 0; jj < groups; ++jj) {
             group(G);
             vp += G * C::PV;
             up += G * C::PU;
@@ -478,19 +480,16 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     };
     // this wavefront's part of a staged stage
     auto compute = [&](int buf_offset, int yl0, int x0) __attribute__((always_inline)) {
-        // groups of G left rows of this stage that can overlap this wavefront's y shifts:
+        // left rows of this stage that can overlap this wavefront's y shifts:
         // rows yl in [syw, syw + TYW - 1 + H - 1] and yl < chi
-        int jj_lo = 0, jj_hi = C::RL / C::G, tail = 0;
+        int row0, nrows;
         {
             int first = syw - yl0;                 // first useful row index j
             int last = syw + C::TYW + H - 2 - yl0; // last useful row index j
             if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
-            if (first > 0) jj_lo = first / C::G;
-            const int rows = last < 0 ? 0 : last + 1; // useful rows from row 0 of the stage
-            if (rows < C::RL) {
-                jj_hi = rows / C::G;
-                tail = rows % C::G;
-            }
+            if (last > C::RL - 1) last = C::RL - 1;
+            row0 = first > 0 ? first : 0;
+            nrows = last + 1 - row0;
         }
         // K-column chunks of this stage that overlap this wavefront's x shifts: need
         // (x0 + kc*K + K-1) + (sxw + TXW-1) >= 0 and (x0 + kc*K) + sxw <= W-1 and x0 + kc*K < W
@@ -504,8 +503,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
             if (h < kc_hi) kc_hi = h;
         }
         if (C::WZ > 1) kc_lo += (group - kc_lo % C::WZ + C::WZ) % C::WZ; // this wavefront's chunks: kc = group (mod WZ)
-        if (jj_lo < jj_hi || (jj_lo == jj_hi && tail > 0))
-            compute_stage<C>(Vs_lane + buf_offset, Us_lane + buf_offset, acc, kc_lo, kc_hi, jj_lo, jj_hi, tail);
+        if (nrows > 0) compute_stage<C>(Vs_lane + buf_offset, Us_lane + buf_offset, acc, kc_lo, kc_hi, row0, nrows / C::G, nrows % C::G);
     };
 
     if constexpr (C::DB) {

@@ -16,6 +16,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "engine.hpp" // vec128
 #include "xcorr_common.hpp"
 
 namespace xcorr {
@@ -327,6 +328,170 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
     rec.rows_per_worker = variant == 2 ? max_rows : rows;
     rec.distribution_type = variant == 2 ? dist : XCORR_DIST_NONE;
     rec.uses_atomics = variant == 2;
+    have_last_launch() = true;
+    return XCORR_OK;
+}
+
+// ------------------------------------------------------------------ whole pair in LDS
+// One small pair (both matrices fit the LDS of a CU together): every block first copies BOTH matrices
+// into LDS - the left one with B zero columns on either side of every row - and then its wavefronts
+// work through tasks of B adjacent x shifts of one output row: lane = right column, per overlapping row
+// one LDS read of the right element and B reads of the left row for B FMAs, the 64 partial sums of a
+// task combined by DPP row operations. One launch, no atomics, no clearing of the output, nothing but
+// LDS traffic after the first 2 * rows * cols * sizeof(T) bytes per block; a 64x64 pair is 4064 tasks,
+// one per wavefront of 256 blocks of 16. This is what the reference's shared-memory warp-per-shift kernel
+// (naive_warp_per_shift_shared_mem.cu:160-420, its fastest at 64x64) reaches for with its row slabs.
+// Tasks are dealt so that the wavefronts of a block get output rows far apart (a mix of long and
+// short overlaps on every CU).
+template <typename T, int B>
+__global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left, const T *__restrict__ right, T *__restrict__ out,
+                                                           int W, int H, int pitch_l, int pitch_r, int tasks_x, int total_tasks) {
+    using vec = typename vec128<T>::type;
+    constexpr int VK = 16 / (int)sizeof(T);
+    constexpr int PAD = B < VK ? VK : B; // zero columns on either side of a left row (keeps 128-bit pieces aligned)
+    extern __shared__ __attribute__((aligned(16))) unsigned char pair_smem[];
+    T *Ls = reinterpret_cast<T *>(pair_smem);
+    T *Rs = Ls + (size_t)H * pitch_l;
+    const int tid = (int)threadIdx.x, nt = (int)blockDim.x;
+    // ---- both matrices into LDS, 128-bit pieces ----
+    {
+        const int pl = pitch_l / VK, pr = pitch_r / VK;
+        for (int p = tid; p < H * pl; p += nt) {
+            const int row = p / pl, col = (p % pl) * VK - PAD; // matrix column of the piece's first element
+            vec v;
+#pragma unroll
+            for (int e = 0; e < VK; ++e) v[e] = T(0);
+            if (col >= 0 && col + VK <= W) {
+                __builtin_memcpy(&v, left + (size_t)row * W + col, sizeof(vec)); // element-aligned only
+            } else {
+#pragma unroll
+                for (int e = 0; e < VK; ++e)
+                    if (col + e >= 0 && col + e < W) v[e] = left[(size_t)row * W + col + e];
+            }
+            *reinterpret_cast<vec *>(Ls + (size_t)p * VK) = v;
+        }
+        for (int p = tid; p < H * pr; p += nt) {
+            const int row = p / pr, col = (p % pr) * VK;
+            vec v;
+#pragma unroll
+            for (int e = 0; e < VK; ++e) v[e] = T(0);
+            if (col + VK <= W) {
+                __builtin_memcpy(&v, right + (size_t)row * W + col, sizeof(vec));
+            } else {
+#pragma unroll
+                for (int e = 0; e < VK; ++e)
+                    if (col + e < W) v[e] = right[(size_t)row * W + col + e];
+            }
+            *reinterpret_cast<vec *>(Rs + (size_t)p * VK) = v;
+        }
+    }
+    __syncthreads();
+    const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
+    const int Sx = 2 * W - 1;
+    // task (wave w of block b, round i) = w * gridDim + b + i * gridDim * nw
+    for (int t = wave * (int)gridDim.x + (int)blockIdx.x; t < total_tasks; t += (int)gridDim.x * nw) {
+        const int oy = t / tasks_x, ox0 = (t % tasks_x) * B;
+        const int sy = oy - (H - 1), sx0 = ox0 - (W - 1);
+        const int y_lo = sy < 0 ? -sy : 0, y_hi = sy > 0 ? H - sy : H;       // right rows that overlap
+        int x_lo = -(sx0 + B - 1), x_hi = W - sx0;                             // right columns that overlap any of the B shifts
+        if (x_lo < 0) x_lo = 0;
+        if (x_hi > W) x_hi = W;
+        T acc[B];
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[b] = T(0);
+        for (int c0 = x_lo; c0 < x_hi; c0 += 64) {
+            const int xr = c0 + lane;
+            if (xr < x_hi) {
+                const T *rp = Rs + (size_t)y_lo * pitch_r + xr;
+                const T *lp = Ls + (size_t)(y_lo + sy) * pitch_l + PAD + xr + sx0;
+                int y = y_lo;
+                // four rows per round: twenty reads in flight ahead of the FMAs that need them
+                for (; y + 4 <= y_hi; y += 4) {
+                    T r[4], l[4][B];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        r[j] = rp[j * pitch_r];
+#pragma unroll
+                        for (int b = 0; b < B; ++b) l[j][b] = lp[j * pitch_l + b];
+                    }
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+#pragma unroll
+                        for (int b = 0; b < B; ++b) acc[b] += l[j][b] * r[j];
+                    rp += 4 * pitch_r;
+                    lp += 4 * pitch_l;
+                }
+                for (; y < y_hi; ++y) {
+                    const T r = *rp;
+#pragma unroll
+                    for (int b = 0; b < B; ++b) acc[b] += lp[b] * r;
+                    rp += pitch_r;
+                    lp += pitch_l;
+                }
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) acc[b] = wave_sum_to_lane63(acc[b]);
+        if (lane == 63) {
+#pragma unroll
+            for (int b = 0; b < B; ++b)
+                if (ox0 + b < Sx) out[(size_t)oy * Sx + ox0 + b] = acc[b];
+        }
+    }
+}
+
+// Bytes of LDS the whole-pair kernel needs for a rows x cols pair (0 when the pair cannot fit).
+template <typename T>
+inline size_t pair_in_lds_bytes(unsigned cols, unsigned rows) {
+    constexpr unsigned VK = 16 / sizeof(T), B = 4, PAD = B < VK ? VK : B;
+    const size_t pitch_l = (cols + 2 * PAD + VK - 1) / VK * VK, pitch_r = (cols + VK - 1) / VK * VK;
+    const size_t bytes = (size_t)rows * (pitch_l + pitch_r) * sizeof(T);
+    return bytes <= 160 * 1024 ? bytes : 0;
+}
+
+template <typename T>
+int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, unsigned cols, unsigned rows, hipStream_t stream) {
+    constexpr unsigned VK = 16 / sizeof(T), B = 4, PAD = B < VK ? VK : B;
+    const size_t bytes = pair_in_lds_bytes<T>(cols, rows);
+    if (bytes == 0) return fail(XCORR_ERR_UNSUPPORTED, "%s: a %u x %u pair does not fit the LDS of a CU", family, rows, cols);
+    const int pitch_l = (int)((cols + 2 * PAD + VK - 1) / VK * VK), pitch_r = (int)((cols + VK - 1) / VK * VK);
+    static bool attr_set[64] = {};
+    int dev = 0;
+    XCORR_HIP(hipGetDevice(&dev));
+    if (bytes > 64 * 1024 && !(dev >= 0 && dev < 64 && attr_set[dev])) {
+        XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, B>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                      160 * 1024));
+        if (dev >= 0 && dev < 64) attr_set[dev] = true;
+    }
+    const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
+    const unsigned tasks_x = (Sx + B - 1) / B, total = tasks_x * Sy;
+    const unsigned waves = 16; // per block
+    unsigned grid = (total + waves - 1) / waves;
+    int cus = 256;
+    {
+        hipDeviceProp_t prop;
+        static int cached = 0;
+        if (cached == 0 && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cached = prop.multiProcessorCount;
+        if (cached > 0) cus = cached;
+    }
+    if (grid > (unsigned)cus) grid = (unsigned)cus; // one block per CU: every block pays for its own copy of the pair
+    pair_in_lds_kernel<T, B><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, (int)cols, (int)rows, pitch_l, pitch_r,
+                                                                              (int)tasks_x, (int)total);
+    XCORR_HIP(hipGetLastError());
+    xcorr_launch_record &rec = last_launch();
+    memset(&rec, 0, sizeof(rec));
+    snprintf(rec.kernel, sizeof(rec.kernel), "%s/pair_in_lds_%s", family, sizeof(T) == 4 ? "f32" : "f64");
+    rec.block[0] = 64 * waves, rec.block[1] = rec.block[2] = 1;
+    rec.grid[0] = grid, rec.grid[1] = rec.grid[2] = 1;
+    rec.shared_mem_bytes = (unsigned)bytes;
+    rec.y_shifts_per_thread = 1;
+    rec.x_shifts_per_thread = B;
+    rec.left_matrices_per_thread = rec.right_matrices_per_thread = 1;
+    rec.lanes_x = rec.lanes_y = 1;
+    rec.rows_per_worker = rows;
+    rec.distribution_type = XCORR_DIST_NONE;
+    rec.blocks_per_cu = 1;
+    rec.column_chunks = 1;
     have_last_launch() = true;
     return XCORR_OK;
 }

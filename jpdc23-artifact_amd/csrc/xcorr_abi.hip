@@ -263,6 +263,17 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     if ((rc = check_limit("shifts per thread", p.shifts_per_thread, Limits::shifts_per_thread))) return rc;
     if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::left_rows))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (p.whole_pair_in_lds > 2) return fail(XCORR_ERR_INVALID_ARGUMENT, "whole_pair_in_lds must be 0, 1 or 2, not %u", p.whole_pair_in_lds);
+    // A small pair with no tile asked for: both matrices in the LDS of every block, one launch, no atomics. Measured
+    // against the engine's best plan on square pairs (microseconds per launch, whole-pair kernel / engine): fp32 16: 3.5 / 5.6,
+    // 32: 4.2 / 7.4, 64: 5.7 / 10.4, 80: 11.1 / 12.6, 96: 15.8 / 16.1, 112: 25.1 / 21.0; fp64 32: 5.2 / 8.0, 64: 8.1 / 13.0,
+    // 80: 15.5 / 17.2, 96: 25.0 / 23.3. Beyond the sizes below the engine's register tiles win.
+    const bool tile_asked = p.specialisation || p.x_shifts_per_thread || p.lanes_x || p.lanes_y || p.rows_per_thread || p.column_chunks ||
+                            p.shifts_per_thread || p.distribution_type != XCORR_DIST_DEFAULT;
+    const size_t elems = (size_t)cols * rows;
+    const bool small = pair_in_lds_bytes<T>(cols, rows) != 0 && cols <= 128 && elems <= (sizeof(T) == 4 ? 96u * 96u : 80u * 80u);
+    if (p.whole_pair_in_lds == 1 || (p.whole_pair_in_lds == 0 && !tile_asked && small))
+        return run_pair_in_lds<T>("grouped_overlap", left, right, out, cols, rows, as_stream(stream));
     EngineRequest rq = base_request("grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = p.shifts_per_thread == 1 ? 2 : p.shifts_per_thread; // 0 = planner's choice among the grouped tiles
     rq.rows_per_worker = p.rows_per_thread;

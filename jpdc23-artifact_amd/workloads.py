@@ -10,7 +10,7 @@ import numpy as np
 
 CONFIGS = {
     "C1": dict(mode="one_to_one", dtype="float32", rows=64, cols=64, n_left=1, n_right=1, dist="uniform", seed=1235,
-               family="warp_per_overlap", params=dict(warp_per_overlap_variant=1, shifts_per_thread_block=4)),
+               family="grouped_overlap"),
     "C2": dict(mode="one_to_one", dtype="float32", rows=1024, cols=1024, n_left=1, n_right=1, dist="uniform", seed=1236,
                family="grouped_overlap"),
     "C3": dict(mode="one_to_many", dtype="float32", rows=256, cols=256, n_left=1, n_right=64, dist="uniform", seed=1237,

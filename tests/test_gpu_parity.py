@@ -60,6 +60,8 @@ ONE_TO_ONE_CASES = [
     ("split_row", dict(distribution_type="triangle", rows_per_thread=4)),
     ("split_row", dict(distribution_type="triangle", rows_per_thread=1)),
     ("grouped_overlap", {}),
+    ("grouped_overlap", dict(whole_pair_in_lds=1)),
+    ("grouped_overlap", dict(whole_pair_in_lds=2)),
     ("grouped_overlap", dict(shifts_per_thread=4, left_rows_per_iteration=3, warps_per_thread_block=8)),
     ("grouped_overlap", dict(shifts_per_thread=8)),
     ("grouped_overlap", dict(shifts_per_thread=1)),
@@ -96,6 +98,50 @@ def test_one_to_one_all_families(oracle, dtype, family, kw):
         exp = oracle.one_to_one(left, right)
         got = xc.run(family, left, right, 1, params=xc.make_params(**kw))
         check(got, exp, False, f"{family} {kw} {shape} real")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_whole_pair_in_lds(oracle, dtype):
+    """The kernel that keeps both matrices of a small pair in LDS (the default of grouped_overlap up to about
+    96 x 96 fp32 / 80 x 80 fp64): every size 1 ... 12 squared, sizes around the 64-column chunk of its lanes,
+    ragged non-square shapes and the largest pairs that fit; bit-exact on integers, within tolerance on real
+    values; the launcher picks it by itself for small pairs and leaves larger ones to the engine; a pair that
+    does not fit is an error when the kernel is forced."""
+    xc = load_package()
+    rng = np.random.default_rng(321)
+    shapes = [(n, n) for n in range(1, 13)] + [(1, 64), (64, 1), (63, 64), (64, 65), (65, 63), (5, 128), (128, 5), (2, 129), (31, 97),
+                                                (80, 80), (96, 96), (90, 101)]
+    shapes += [(128, 128), (136, 130)] if dtype == np.float32 else [(100, 97)]
+    for shape in shapes:
+        say("whole pair in LDS", np.dtype(dtype).name, shape)
+        left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
+        got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=1))
+        assert "pair_in_lds" in xc.last_launch()["kernel"]
+        assert xc.last_launch()["uses_atomics"] == 0
+        check(got, oracle.one_to_one(left, right), True, f"whole pair {shape} int")
+        left, right = rng.standard_normal(shape).astype(dtype), rng.random(shape).astype(dtype)
+        got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=1))
+        check(got, oracle.one_to_one(left, right), False, f"whole pair {shape} real")
+    # the launcher's own choice
+    for shape, expect in [((64, 64), True), ((40, 90), True), ((200, 200), False), ((3, 300), False)]:
+        left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
+        got = xc.run("grouped_overlap", left, right, 1)
+        assert ("pair_in_lds" in xc.last_launch()["kernel"]) == expect, (shape, xc.last_launch()["kernel"])
+        check(got, oracle.one_to_one(left, right), True, f"default {shape}")
+        got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=2))
+        assert "pair_in_lds" not in xc.last_launch()["kernel"]
+        check(got, oracle.one_to_one(left, right), True, f"engine {shape}")
+    # asking for a tile keeps the engine
+    left, right = ints(rng, (32, 32), dtype), ints(rng, (32, 32), dtype)
+    xc.run("grouped_overlap", left, right, 1, params=xc.make_params(shifts_per_thread=4))
+    assert "pair_in_lds" not in xc.last_launch()["kernel"]
+    big = (300, 300)
+    with pytest.raises(xc.XcorrError) as err:
+        xc.run("grouped_overlap", ints(rng, big, dtype), ints(rng, big, dtype), 1, params=xc.make_params(whole_pair_in_lds=1))
+    assert err.value.code == 3 and "does not fit" in err.value.message
+    with pytest.raises(xc.XcorrError) as err:
+        xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=3))
+    assert err.value.code == 1
 
 
 ONE_TO_MANY_CASES = [
