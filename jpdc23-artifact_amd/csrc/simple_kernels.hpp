@@ -334,158 +334,203 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
 
 // ------------------------------------------------------------------ whole pair in LDS
 // One small pair (both matrices fit the LDS of a CU together): every block first copies BOTH matrices
-// into LDS - the left one with B zero columns on either side of every row - and then its wavefronts
-// work through tasks of B adjacent x shifts of one output row: lane = right column, per overlapping row
-// one LDS read of the right element and B reads of the left row for B FMAs, the 64 partial sums of a
-// task combined by DPP row operations. One launch, no atomics, no clearing of the output, nothing but
-// LDS traffic after the first 2 * rows * cols * sizeof(T) bytes per block; a 64x64 pair is 4064 tasks,
-// one per wavefront of 256 blocks of 16. This is what the reference's shared-memory warp-per-shift kernel
-// (naive_warp_per_shift_shared_mem.cu:160-420, its fastest at 64x64) reaches for with its row slabs.
-// Tasks are dealt so that the wavefronts of a block get output rows far apart (a mix of long and
-// short overlaps on every CU).
-template <typename T, int B>
+// into LDS - the left one with B zero columns on either side of every row and a few zero rows above and
+// below, the right one with zero rows below - and then its wavefronts work through tasks of A adjacent
+// y shifts x B adjacent x shifts: lane = right column; per overlapping right row one LDS read of the right
+// element and B reads of ONE new left row (the A left rows a step pairs with that right row slide down by
+// one row per step and are kept in registers) for A * B FMAs; the 64 partial sums of every shift are
+// combined by DPP row operations. One launch, no atomics, no clearing of the output, nothing but LDS
+// traffic after the first 2 * rows * cols * sizeof(T) bytes per block; a 64x64 fp32 pair is 4064 tasks of one
+// y shift, one per wavefront of 256 blocks of 16. This is what the reference's shared-memory
+// warp-per-shift kernel (naive_warp_per_shift_shared_mem.cu:160-420, its fastest at 64x64) reaches for with
+// its row slabs. Tasks are dealt so that the wavefronts of a block get output rows far apart (a mix of
+// long and short overlaps on every CU).
+template <typename T, int A, int B, int U>
 __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left, const T *__restrict__ right, T *__restrict__ out,
                                                            int W, int H, int pitch_l, int pitch_r, int tasks_x, int total_tasks) {
     using vec = typename vec128<T>::type;
     constexpr int VK = 16 / (int)sizeof(T);
-    constexpr int PAD = B < VK ? VK : B; // zero columns on either side of a left row (keeps 128-bit pieces aligned)
+    constexpr int PAD = B < VK ? VK : B;          // zero columns on either side of a left row (keeps 128-bit pieces aligned)
+    constexpr int TOP = A - 1, BOT = U + A - 2;   // zero rows above / below the left matrix; the right one has U - 1 below
     extern __shared__ __attribute__((aligned(16))) unsigned char pair_smem[];
     T *Ls = reinterpret_cast<T *>(pair_smem);
-    T *Rs = Ls + (size_t)H * pitch_l;
+    const int rows_l = H + TOP + BOT, rows_r = H + U - 1;
+    T *Rs = Ls + (size_t)rows_l * pitch_l;
     const int tid = (int)threadIdx.x, nt = (int)blockDim.x;
-    // ---- both matrices into LDS, 128-bit pieces ----
+    // ---- both matrices into LDS, 128-bit pieces; the loads of four pieces per thread are in flight together ----
     {
         const int pl = pitch_l / VK, pr = pitch_r / VK;
-        for (int p = tid; p < H * pl; p += nt) {
-            const int row = p / pl, col = (p % pl) * VK - PAD; // matrix column of the piece's first element
-            vec v;
+        const int total_l = rows_l * pl, total = total_l + rows_r * pr; // the right image follows the left one
+        constexpr int NB = 4;
+        for (int p0 = tid; p0 < total; p0 += nt * NB) {
+            vec v[NB];
 #pragma unroll
-            for (int e = 0; e < VK; ++e) v[e] = T(0);
-            if (col >= 0 && col + VK <= W) {
-                __builtin_memcpy(&v, left + (size_t)row * W + col, sizeof(vec)); // element-aligned only
-            } else {
+            for (int j = 0; j < NB; ++j) {
+                const int p = p0 + j * nt;
 #pragma unroll
-                for (int e = 0; e < VK; ++e)
-                    if (col + e >= 0 && col + e < W) v[e] = left[(size_t)row * W + col + e];
+                for (int e = 0; e < VK; ++e) v[j][e] = T(0);
+                if (p >= total) continue;
+                const bool is_left = p < total_l;
+                const int q = is_left ? p : p - total_l, pp = is_left ? pl : pr;
+                const int row = q / pp - (is_left ? TOP : 0), col = (q % pp) * VK - (is_left ? PAD : 0); // matrix row, first column
+                if (row < 0 || row >= H) continue;
+                const T *src = (is_left ? left : right) + (size_t)row * W + col;
+                if (col >= 0 && col + VK <= W) {
+                    __builtin_memcpy(&v[j], src, sizeof(vec)); // element-aligned only
+                } else {
+#pragma unroll
+                    for (int e = 0; e < VK; ++e)
+                        if (col + e >= 0 && col + e < W) v[j][e] = src[e];
+                }
             }
-            *reinterpret_cast<vec *>(Ls + (size_t)p * VK) = v;
-        }
-        for (int p = tid; p < H * pr; p += nt) {
-            const int row = p / pr, col = (p % pr) * VK;
-            vec v;
 #pragma unroll
-            for (int e = 0; e < VK; ++e) v[e] = T(0);
-            if (col + VK <= W) {
-                __builtin_memcpy(&v, right + (size_t)row * W + col, sizeof(vec));
-            } else {
-#pragma unroll
-                for (int e = 0; e < VK; ++e)
-                    if (col + e < W) v[e] = right[(size_t)row * W + col + e];
+            for (int j = 0; j < NB; ++j) {
+                const int p = p0 + j * nt;
+                if (p < total) *reinterpret_cast<vec *>(Ls + (size_t)p * VK) = v[j];
             }
-            *reinterpret_cast<vec *>(Rs + (size_t)p * VK) = v;
         }
     }
     __syncthreads();
     const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
-    const int Sx = 2 * W - 1;
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     // task (wave w of block b, round i) = w * gridDim + b + i * gridDim * nw
     for (int t = wave * (int)gridDim.x + (int)blockIdx.x; t < total_tasks; t += (int)gridDim.x * nw) {
-        const int oy = t / tasks_x, ox0 = (t % tasks_x) * B;
-        const int sy = oy - (H - 1), sx0 = ox0 - (W - 1);
-        const int y_lo = sy < 0 ? -sy : 0, y_hi = sy > 0 ? H - sy : H;       // right rows that overlap
-        int x_lo = -(sx0 + B - 1), x_hi = W - sx0;                             // right columns that overlap any of the B shifts
+        const int oy0 = (t / tasks_x) * A, ox0 = (t % tasks_x) * B;
+        const int sy0 = oy0 - (H - 1), sx0 = ox0 - (W - 1);
+        // right rows / columns that overlap any of the A x B shifts
+        int y_lo = -(sy0 + A - 1), y_hi = H - sy0, x_lo = -(sx0 + B - 1), x_hi = W - sx0;
+        if (y_lo < 0) y_lo = 0;
+        if (y_hi > H) y_hi = H;
         if (x_lo < 0) x_lo = 0;
         if (x_hi > W) x_hi = W;
-        T acc[B];
+        const int rounds = (y_hi - y_lo + U - 1) / U; // whole rounds of U rows: the last one may run into the zero rows
+        T acc[A][B];
 #pragma unroll
-        for (int b = 0; b < B; ++b) acc[b] = T(0);
+        for (int a = 0; a < A; ++a)
+#pragma unroll
+            for (int b = 0; b < B; ++b) acc[a][b] = T(0);
         for (int c0 = x_lo; c0 < x_hi; c0 += 64) {
             const int xr = c0 + lane;
             if (xr < x_hi) {
                 const T *rp = Rs + (size_t)y_lo * pitch_r + xr;
-                const T *lp = Ls + (size_t)(y_lo + sy) * pitch_l + PAD + xr + sx0;
-                int y = y_lo;
-                // four rows per round: twenty reads in flight ahead of the FMAs that need them
-                for (; y + 4 <= y_hi; y += 4) {
-                    T r[4], l[4][B];
+                const T *lp = Ls + (size_t)(y_lo + sy0 + TOP) * pitch_l + PAD + xr + sx0; // left row that pairs with y_lo for shift sy0
+                // left rows y + sy0 .. y + sy0 + U + A - 2 of a round that starts at right row y; the last A - 1 of them
+                // are the first A - 1 of the next round
+                T win[U + A - 1][B];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
+                for (int a = 0; a < A - 1; ++a)
+#pragma unroll
+                    for (int b = 0; b < B; ++b) win[a][b] = lp[a * pitch_l + b];
+                for (int g = 0; g < rounds; ++g) {
+                    T r[U];
+#pragma unroll
+                    for (int j = 0; j < U; ++j) { // U * (B + 1) reads in flight ahead of the FMAs
                         r[j] = rp[j * pitch_r];
 #pragma unroll
-                        for (int b = 0; b < B; ++b) l[j][b] = lp[j * pitch_l + b];
+                        for (int b = 0; b < B; ++b) win[A - 1 + j][b] = lp[(A - 1 + j) * pitch_l + b];
                     }
 #pragma unroll
-                    for (int j = 0; j < 4; ++j)
+                    for (int j = 0; j < U; ++j)
 #pragma unroll
-                        for (int b = 0; b < B; ++b) acc[b] += l[j][b] * r[j];
-                    rp += 4 * pitch_r;
-                    lp += 4 * pitch_l;
-                }
-                for (; y < y_hi; ++y) {
-                    const T r = *rp;
+                        for (int a = 0; a < A; ++a)
 #pragma unroll
-                    for (int b = 0; b < B; ++b) acc[b] += lp[b] * r;
-                    rp += pitch_r;
-                    lp += pitch_l;
+                            for (int b = 0; b < B; ++b) acc[a][b] += win[j + a][b] * r[j];
+#pragma unroll
+                    for (int a = 0; a < A - 1; ++a)
+#pragma unroll
+                        for (int b = 0; b < B; ++b) win[a][b] = win[U + a][b];
+                    rp += U * pitch_r;
+                    lp += U * pitch_l;
                 }
             }
         }
 #pragma unroll
-        for (int b = 0; b < B; ++b) acc[b] = wave_sum_to_lane63(acc[b]);
+        for (int a = 0; a < A; ++a)
+#pragma unroll
+            for (int b = 0; b < B; ++b) acc[a][b] = wave_sum_to_lane63(acc[a][b]);
         if (lane == 63) {
 #pragma unroll
-            for (int b = 0; b < B; ++b)
-                if (ox0 + b < Sx) out[(size_t)oy * Sx + ox0 + b] = acc[b];
+            for (int a = 0; a < A; ++a)
+#pragma unroll
+                for (int b = 0; b < B; ++b)
+                    if (oy0 + a < Sy && ox0 + b < Sx) out[(size_t)(oy0 + a) * Sx + ox0 + b] = acc[a][b];
         }
     }
 }
 
-// Bytes of LDS the whole-pair kernel needs for a rows x cols pair (0 when the pair cannot fit).
+constexpr int PAIR_B = 4; // x shifts per task of the whole-pair kernel
+
+// Bytes of LDS the whole-pair kernel needs for a rows x cols pair with A y shifts per task and U rows per round.
 template <typename T>
-inline size_t pair_in_lds_bytes(unsigned cols, unsigned rows) {
-    constexpr unsigned VK = 16 / sizeof(T), B = 4, PAD = B < VK ? VK : B;
+inline size_t pair_in_lds_bytes(unsigned cols, unsigned rows, unsigned A, unsigned U) {
+    constexpr unsigned VK = 16 / sizeof(T), PAD = PAIR_B < VK ? VK : PAIR_B;
     const size_t pitch_l = (cols + 2 * PAD + VK - 1) / VK * VK, pitch_r = (cols + VK - 1) / VK * VK;
-    const size_t bytes = (size_t)rows * (pitch_l + pitch_r) * sizeof(T);
-    return bytes <= 160 * 1024 ? bytes : 0;
+    return ((size_t)(rows + U + 2 * A - 3) * pitch_l + (size_t)(rows + U - 1) * pitch_r) * sizeof(T);
+}
+// whether the whole-pair kernel can run a rows x cols pair at all (its smallest variant)
+template <typename T>
+inline bool pair_fits_lds(unsigned cols, unsigned rows) {
+    return pair_in_lds_bytes<T>(cols, rows, 2, 4) <= 160 * 1024;
 }
 
-template <typename T>
-int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, unsigned cols, unsigned rows, hipStream_t stream) {
-    constexpr unsigned VK = 16 / sizeof(T), B = 4, PAD = B < VK ? VK : B;
-    const size_t bytes = pair_in_lds_bytes<T>(cols, rows);
-    if (bytes == 0) return fail(XCORR_ERR_UNSUPPORTED, "%s: a %u x %u pair does not fit the LDS of a CU", family, rows, cols);
+template <typename T, int A, int U>
+int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, unsigned rows, size_t bytes, unsigned *grid_out,
+                       unsigned *waves_out, hipStream_t stream) {
+    constexpr unsigned VK = 16 / sizeof(T), B = PAIR_B, PAD = B < VK ? VK : B;
     const int pitch_l = (int)((cols + 2 * PAD + VK - 1) / VK * VK), pitch_r = (int)((cols + VK - 1) / VK * VK);
     static bool attr_set[64] = {};
     int dev = 0;
     XCORR_HIP(hipGetDevice(&dev));
     if (bytes > 64 * 1024 && !(dev >= 0 && dev < 64 && attr_set[dev])) {
-        XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, B>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, A, B, U>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024));
         if (dev >= 0 && dev < 64) attr_set[dev] = true;
     }
     const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
-    const unsigned tasks_x = (Sx + B - 1) / B, total = tasks_x * Sy;
-    const unsigned waves = 16; // per block
-    unsigned grid = (total + waves - 1) / waves;
-    int cus = 256;
-    {
+    const unsigned tasks_x = (Sx + B - 1) / B, total = tasks_x * ((Sy + A - 1) / A);
+    static int cus = 0;
+    if (cus == 0) {
         hipDeviceProp_t prop;
-        static int cached = 0;
-        if (cached == 0 && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cached = prop.multiProcessorCount;
-        if (cached > 0) cus = cached;
+        cus = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
     }
+    // eight wavefronts per block while that still gives every task a wavefront of its own, else sixteen
+    const unsigned waves = total <= 8u * (unsigned)cus ? 8 : 16;
+    unsigned grid = (total + waves - 1) / waves;
     if (grid > (unsigned)cus) grid = (unsigned)cus; // one block per CU: every block pays for its own copy of the pair
-    pair_in_lds_kernel<T, B><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, (int)cols, (int)rows, pitch_l, pitch_r,
-                                                                              (int)tasks_x, (int)total);
+    pair_in_lds_kernel<T, A, B, U><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, (int)cols, (int)rows, pitch_l, pitch_r,
+                                                                                    (int)tasks_x, (int)total);
     XCORR_HIP(hipGetLastError());
+    *grid_out = grid;
+    *waves_out = waves;
+    return XCORR_OK;
+}
+
+template <typename T>
+int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, unsigned cols, unsigned rows, hipStream_t stream) {
+    if (!pair_fits_lds<T>(cols, rows)) return fail(XCORR_ERR_UNSUPPORTED, "%s: a %u x %u pair does not fit the LDS of a CU", family, rows, cols);
+    // One y shift per task while the tasks are few (at 64x64 fp32 every wavefront slot of the device gets one task: the
+    // kernel is bound by the latency of a task, not by LDS throughput), two beyond. Measured, microseconds per launch with
+    // one / two y shifts per task: fp32 64x64 6.0 / 6.8, 96x96 17.0 / 14.1, 128x128 46 / 29; fp64 32x32 4.4 / 5.0,
+    // 64x64 9.0 / 8.6, 96x96 27 / 19. Eight rows per round instead of four changed nothing.
+    constexpr unsigned U = 4;
+    unsigned A = (size_t)cols * rows <= (sizeof(T) == 4 ? 88u * 88u : 40u * 40u) ? 1 : 2;
+    if (pair_in_lds_bytes<T>(cols, rows, A, U) > 160 * 1024) A = 2;
+    const size_t bytes = pair_in_lds_bytes<T>(cols, rows, A, U);
+    unsigned grid = 0, waves = 0;
+    int rc;
+    if (A == 1)
+        rc = launch_pair_in_lds<T, 1, U>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else
+        rc = launch_pair_in_lds<T, 2, U>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    if (rc != XCORR_OK) return rc;
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
-    snprintf(rec.kernel, sizeof(rec.kernel), "%s/pair_in_lds_%s", family, sizeof(T) == 4 ? "f32" : "f64");
+    snprintf(rec.kernel, sizeof(rec.kernel), "%s/pair_in_lds_%s_a%u", family, sizeof(T) == 4 ? "f32" : "f64", A);
     rec.block[0] = 64 * waves, rec.block[1] = rec.block[2] = 1;
     rec.grid[0] = grid, rec.grid[1] = rec.grid[2] = 1;
     rec.shared_mem_bytes = (unsigned)bytes;
-    rec.y_shifts_per_thread = 1;
-    rec.x_shifts_per_thread = B;
+    rec.y_shifts_per_thread = A;
+    rec.x_shifts_per_thread = PAIR_B;
     rec.left_matrices_per_thread = rec.right_matrices_per_thread = 1;
     rec.lanes_x = rec.lanes_y = 1;
     rec.rows_per_worker = rows;

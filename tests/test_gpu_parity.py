@@ -102,8 +102,8 @@ def test_one_to_one_all_families(oracle, dtype, family, kw):
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_whole_pair_in_lds(oracle, dtype):
-    """The kernel that keeps both matrices of a small pair in LDS (the default of grouped_overlap up to about
-    96 x 96 fp32 / 80 x 80 fp64): every size 1 ... 12 squared, sizes around the 64-column chunk of its lanes,
+    """The kernel that keeps both matrices of a small pair in LDS (the default of grouped_overlap up to
+    112 x 112 fp32 / 96 x 96 fp64): every size 1 ... 12 squared, sizes around the 64-column chunk of its lanes,
     ragged non-square shapes and the largest pairs that fit; bit-exact on integers, within tolerance on real
     values; the launcher picks it by itself for small pairs and leaves larger ones to the engine; a pair that
     does not fit is an error when the kernel is forced."""
@@ -111,7 +111,7 @@ def test_whole_pair_in_lds(oracle, dtype):
     rng = np.random.default_rng(321)
     shapes = [(n, n) for n in range(1, 13)] + [(1, 64), (64, 1), (63, 64), (64, 65), (65, 63), (5, 128), (128, 5), (2, 129), (31, 97),
                                                 (80, 80), (96, 96), (90, 101)]
-    shapes += [(128, 128), (136, 130)] if dtype == np.float32 else [(100, 97)]
+    shapes += [(128, 128), (136, 130)] if dtype == np.float32 else [(98, 94)]
     for shape in shapes:
         say("whole pair in LDS", np.dtype(dtype).name, shape)
         left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
@@ -123,7 +123,7 @@ def test_whole_pair_in_lds(oracle, dtype):
         got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=1))
         check(got, oracle.one_to_one(left, right), False, f"whole pair {shape} real")
     # the launcher's own choice
-    for shape, expect in [((64, 64), True), ((40, 90), True), ((200, 200), False), ((3, 300), False)]:
+    for shape, expect in [((64, 64), True), ((40, 90), True), ((110, 100), np.dtype(dtype) == np.float32), ((200, 200), False), ((3, 300), False)]:
         left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
         got = xc.run("grouped_overlap", left, right, 1)
         assert ("pair_in_lds" in xc.last_launch()["kernel"]) == expect, (shape, xc.last_launch()["kernel"])
