@@ -57,12 +57,19 @@ extern "C" {
  * Tuning integers, named after the reference's per-algorithm JSON keys
  * (one_to_one.hpp:739-741, n_to_m.hpp:321-325, n_to_m.hpp:475-479, ...). The
  * reference counts 32-lane warps and instantiates one kernel per value; this
- * library runs a short list of gfx950 tiles on 64-lane wavefronts and picks the one
- * its cost model rates best for the sizes at hand. The integers are checked against
- * the reference's release limits (CMakeLists.txt:16-46; larger values are rejected
- * as there) and otherwise only break ties between equally rated tiles; the tile
- * actually used is reported by xcorr_last_launch(). The geometry fields further down
- * select a tile exactly.
+ * library runs a short list of gfx950 tiles on 64-lane wavefronts. All integers are
+ * checked against the reference's release limits (CMakeLists.txt:16-46; larger
+ * values are rejected as there). 0 leaves a choice to the library's cost model.
+ * A non-zero shifts_per_thread / shifts_per_thread_right_matrix,
+ * right_matrices_per_thread or left_matrices_per_thread is an exact request: the
+ * launch uses the compiled tile with the nearest value at or above it (y shifts per
+ * lane: 4 or 8; matrices per lane position = matrices per lane x lanes laid over
+ * matrices: 1, 4, 8, 16; the distances of the three requests add up), and among
+ * equally near tiles the one the cost model rates fastest. left_rows_per_iteration and
+ * warps_per_thread_block have no counterpart in these kernels (every tile stages its
+ * own band height and runs four wavefronts per block) and are only validated.
+ * The tile actually used is reported by xcorr_last_launch(). The geometry fields
+ * further down select a tile exactly.
  */
 typedef struct xcorr_params {
     unsigned warps_per_thread_block;         /* <= 32 */

@@ -25,8 +25,6 @@ static int device_cus() {
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)); }
-
 // Relative cost of running a request of the one-output-row families on one of their tiles
 // (their four wavefronts tile 2x2 over the shifts):
 //   * work issued for partial overlaps at tile edges: a wavefront skips what cannot overlap its
@@ -36,7 +34,6 @@ static double log2_ratio(double a, double b) { return std::fabs(std::log2(a / b)
 //   * issue slots lost to LDS reads (a read plus the wait that guards it displace about nine fp32
 //     FMA slots, half as many fp64 ones);
 //   * several matrices per lane: the register ring of right rows grows, some spills.
-// The reference's tuning integers only break ties (2 % per doubling away from the request).
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
     double waste_y = std::sqrt((double)(rq.H + s.TYW()) * (rq.H + s.TYB())) / rq.H;
@@ -49,10 +46,28 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
     cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
     if (s.NV * s.NU > 1) cost *= 1.15;
-    if (rq.left_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NV * s.LV, rq.left_mats);
-    if (rq.right_mats) cost *= 1.0 + 0.02 * log2_ratio(s.NU * s.LU, rq.right_mats);
-    if (rq.waves) cost *= 1.0 + 0.01 * log2_ratio(s.WX * s.WY * s.WZ, rq.waves);
     return cost;
+}
+
+// How far a tile's value x is from a requested tuning integer r (0: not requested): nothing when it matches, the number
+// of doublings above the request when the tile has more, and a large penalty when it has fewer (the nearest compiled
+// value at or above the request is wanted; if none exists the largest below it).
+static double request_distance(int x, unsigned r) {
+    if (r == 0) return 0.0;
+    return x >= (int)r ? std::log2((double)x / r) : 16.0 + std::log2((double)r / x);
+}
+
+// The reference's tuning integers, when given (non-zero), are exact requests: the tile must come as close as the compiled
+// list allows to `y_shifts` adjacent y shifts per lane and to `right_mats` / `left_mats` matrices per lane position
+// (matrices per lane x lanes laid over matrices). The distances add up; the sum is compared before any cost or run time.
+struct RequestMatch {
+    double d;
+    bool better_than(const RequestMatch &o) const { return d < o.d; }
+    bool same_as(const RequestMatch &o) const { return d == o.d; }
+};
+static RequestMatch match_request(const EngineSpec &s, const EngineRequest &rq) {
+    return RequestMatch{(s.A > 1 ? request_distance(s.A, rq.y_shifts > 1 ? rq.y_shifts : 0) : 0.0) + request_distance(s.NUB(), rq.right_mats) +
+                        request_distance(s.NVB(), rq.left_mats)};
 }
 
 // Number of (y tile, chunk) workers when every y tile's rows are cut into chunks of rc rows.
@@ -184,11 +199,12 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
 
 // Grouped families: every compatible tile is tried with the reduction uncut and cut into 2, 3, 4, 6 ...
 // groups of G = A + 1 rows (the granule of the inner loop); the plan with the shortest predicted
-// run time wins. The reference's tuning integers only break ties (0.5 % per doubling away).
+// run time wins among the tiles that match the reference's tuning integers best (match_request; all tiles when none is given).
 static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int count, EnginePlan &plan) {
     static const int ladder[] = {0, 2, 3, 4, 6, 8, 12, 16, 24, 32};
     bool found = false;
     double best = 0;
+    RequestMatch best_match = {};
     for (int i = 0; i < count; ++i) {
         const EngineSpec &s = specs[i];
         if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
@@ -198,6 +214,8 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
             if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
             if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
         }
+        const RequestMatch match = match_request(s, rq);
+        if (found && best_match.better_than(match)) continue;
         const int G = s.A + 1;
         for (int k : ladder) {
             int rc = k * G;
@@ -211,13 +229,11 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
             }
             EnginePlan cand;
             if (int e = shape_plan(s, rq, rc, (int)rq.column_chunks, cand)) return e;
-            double t = predict_us(s, rq, cand);
-            if (rq.y_shifts > 1) t *= 1.0 + 0.005 * log2_ratio(s.A, rq.y_shifts);
-            if (rq.left_mats) t *= 1.0 + 0.005 * log2_ratio(s.NV * s.LV, rq.left_mats);
-            if (rq.right_mats) t *= 1.0 + 0.005 * log2_ratio(s.NU * s.LU, rq.right_mats);
-            if (!found || t < best) {
+            const double t = predict_us(s, rq, cand);
+            if (!found || match.better_than(best_match) || t < best) {
                 found = true;
                 best = t;
+                best_match = match;
                 plan = cand;
             }
         }
@@ -250,6 +266,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     // one-output-row families: relative cost of the tile, then the split rule below
     const EngineSpec *best = rq.spec_index > 0 ? &specs[rq.spec_index - 1] : nullptr;
     double best_cost = 0;
+    RequestMatch best_match = {};
     for (int i = 0; i < count && rq.spec_index == 0; ++i) {
         const EngineSpec &s = specs[i];
         if (s.A != 1) continue;
@@ -257,10 +274,12 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
         if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
         if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
-        double c = spec_cost(s, rq);
-        if (!best || c < best_cost) {
+        const double c = spec_cost(s, rq);
+        const RequestMatch match = match_request(s, rq);
+        if (!best || match.better_than(best_match) || (match.same_as(best_match) && c < best_cost)) {
             best = &s;
             best_cost = c;
+            best_match = match;
         }
     }
     if (!best)

@@ -99,9 +99,10 @@ std::vector<algorithm_def> build_defs() {
         std::vector<A> v = mrg;
         v.push_back(streams());
         auto &a = add("nai_shuffle_multirow_both_multimat_right_n_to_mn", Mode::n_to_mn, Family::multimat_right_grouped, v);
-        // one launch over all left matrices instead of the reference's launch per left matrix on
-        // num_cuda_streams streams (n_to_mn.hpp:553-571): the key is read and reported, not used
+        // one launch over all left matrices by default; when the arguments file holds num_cuda_streams, one launch per
+        // left matrix on that many streams like the reference (n_to_mn.hpp:553-571)
         a.deinterleave = true;
+        a.per_left_streams_if_asked = true;
     }
     // multi-matrix-both x grouped-overlap (n_to_m.hpp:470)
     add("nai_shuffle_multirow_both_multimat_both_n_to_m", Mode::n_to_m, Family::multimat_both_grouped,
@@ -125,7 +126,8 @@ std::vector<algorithm_def> build_defs() {
         std::vector<A> v = mrr;
         v.push_back(streams());
         auto &a = add("nai_shuffle_multirow_right_multimat_right_n_to_mn", Mode::n_to_mn, Family::multimat_right_grouped, v);
-        a.deinterleave = true; // one launch, as above
+        a.deinterleave = true; // one launch unless num_cuda_streams is given, as above
+        a.per_left_streams_if_asked = true;
     }
     // warp-per-overlap (one_to_one.hpp:410, :519, :452)
     add("nai_warp_per_shift_one_to_one", Mode::one_to_one, Family::warp_per_overlap,
@@ -228,6 +230,14 @@ std::optional<Mode> parse_mode(const std::string &name) {
 }
 
 // ---------------------------------------------------------------- gpu_algorithm
+namespace {
+// keys whose value picks a compiled tile in the library: an exact request there, so only passed when the file holds them
+bool selects_tile(const std::string &key) {
+    return key == "shifts_per_thread" || key == "shifts_per_thread_right_matrix" || key == "right_rows_per_thread" ||
+           key == "right_matrices_per_thread" || key == "left_matrices_per_thread";
+}
+} // namespace
+
 template <typename T>
 gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args, BenchmarkType bench, std::chrono::nanoseconds min_time)
     : algorithm(bench, 1, min_time), def_(def) {
@@ -254,7 +264,7 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
             if (std::string(a.key) == "num_cuda_streams") num_streams_ = value;
             shown = std::to_string(value);
         }
-        if (a.field) params_.*(a.field) = value;
+        if (a.field) params_.*(a.field) = selects_tile(a.key) && !args.contains(a.key) ? 0u : value;
         if (a.report) props_.emplace_back(a.key, shown);
     }
     if (def.shared_mem_rows_rule && shared_mem_rows < shifts_per_thread_block) {
@@ -266,7 +276,8 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
     // (the shifts-per-block and block-size limits are the launchers': they fail in the first launch, exit code 3)
     zero_output_ = def.zero_output || (def.family == Family::warp_per_overlap_lds && params_.column_group_per_block);
     if (def.fixed_one_right_per_thread) params_.right_matrices_per_thread = 1;
-    if (def.per_left_streams && num_streams_ == 0) num_streams_ = 1;
+    if (def.per_left_streams_if_asked && args.contains("num_cuda_streams")) def_.per_left_streams = true;
+    if (def_.per_left_streams && num_streams_ == 0) num_streams_ = 1;
     // the unpublished "multirow_right" kernels allow up to 8 rows, the combined engine tiles 4
     if (def.family == Family::multimat_right_grouped && params_.shifts_per_thread_right_matrix > 4 &&
         def.name.find("multirow_right") != std::string::npos)
@@ -274,9 +285,19 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
 }
 
 template <typename T>
+void gpu_algorithm<T>::release() noexcept {
+    for (auto &s : streams_)
+        if (s) xcorr_stream_destroy(s);
+    streams_.clear();
+    if (d_results_) xcorr_free(d_results_);
+    if (d_targets_) xcorr_free(d_targets_);
+    if (d_refs_) xcorr_free(d_refs_);
+    d_results_ = d_targets_ = d_refs_ = nullptr;
+}
+
+template <typename T>
 gpu_algorithm<T>::~gpu_algorithm() {
-    // buffers and streams are released in free(); nothing is left when a phase threw before that
-    // except device memory the process is about to give back anyway
+    release(); // whatever a phase that threw left behind (free() has released everything after a normal run)
 }
 
 template <typename T>
@@ -347,10 +368,7 @@ void gpu_algorithm<T>::launch_all() {
         for (dsize_t r = 0; r < n; ++r) {
             const T *right = all_pairs ? d_targets_ : d_targets_ + (std::size_t)r * per_left * in_area;
             T *out = d_results_ + (std::size_t)r * per_left * out_area;
-            if (def_.family == Family::overlap_wise)
-                launch(d_refs_ + r * in_area, right, out, 1, per_left, streams_[r % streams_.size()]);
-            else
-                launch(d_refs_ + r * in_area, right, out, 1, per_left, streams_[r % streams_.size()]);
+            launch(d_refs_ + r * in_area, right, out, 1, per_left, streams_[r % streams_.size()]);
         }
         return;
     }
@@ -373,6 +391,23 @@ void gpu_algorithm<T>::run_impl() {
     } else {
         sw_.device_adaptive_measure(0, measure_alg(), [&] { launch_all(); });
     }
+    report_effective_arguments();
+}
+
+// The measurement file reports what the launch used, not what was asked: the library maps the reference's integers onto
+// its compiled tiles (xcorr_last_launch).
+template <typename T>
+void gpu_algorithm<T>::report_effective_arguments() {
+    xcorr_launch_record rec;
+    if (xcorr_last_launch(&rec) != XCORR_OK) return;
+    for (auto &[key, value] : props_) {
+        if (key == "shifts_per_thread" || key == "shifts_per_thread_right_matrix" || key == "right_rows_per_thread")
+            value = std::to_string(rec.y_shifts_per_thread);
+        else if (key == "right_matrices_per_thread")
+            value = std::to_string(rec.right_matrices_per_thread * (rec.lanes_right ? rec.lanes_right : 1u));
+        else if (key == "left_matrices_per_thread")
+            value = std::to_string(rec.left_matrices_per_thread * (rec.lanes_left ? rec.lanes_left : 1u));
+    }
 }
 
 template <typename T>
@@ -382,12 +417,15 @@ void gpu_algorithm<T>::finalize_impl() {
 
 template <typename T>
 void gpu_algorithm<T>::free_impl() {
-    for (auto &s : streams_) xcheck(xcorr_stream_destroy(s));
+    for (auto &s : streams_) {
+        void *stream = s;
+        s = nullptr;
+        xcheck(xcorr_stream_destroy(stream));
+    }
     streams_.clear();
-    xcheck(xcorr_free(d_results_));
-    xcheck(xcorr_free(d_targets_));
-    xcheck(xcorr_free(d_refs_));
+    T *buffers[3] = {d_results_, d_targets_, d_refs_};
     d_results_ = d_targets_ = d_refs_ = nullptr;
+    for (T *b : buffers) xcheck(xcorr_free(b));
 }
 
 template <typename T>

@@ -197,6 +197,9 @@ enum class Family {
 // One JSON key of an algorithm: its default, the xcorr_params field it feeds (may be none for
 // keys that only exist for drop-in compatibility) and whether it is a fixed value that is
 // reported but not read.
+// The integers that pick a compiled tile in the library (shifts / matrices per thread) are exact requests there: they
+// are passed only when the arguments file holds the key, 0 (the library's own choice) otherwise, and the measurement
+// file reports the values the launch really used.
 struct arg_spec {
     enum class type { uint, boolean, distribution };
     const char *key;
@@ -212,6 +215,7 @@ struct algorithm_def {
     Family family;
     std::vector<arg_spec> args;
     bool per_left_streams = false; // one launch per left matrix, round robin over num_cuda_streams
+    bool per_left_streams_if_asked = false; // the same, but only when the arguments file holds num_cuda_streams
     bool deinterleave = false;     // n_to_mn: right matrices grouped per left matrix on the device
     bool zero_output = false;      // split-row contract: clear the output inside the measured block
     unsigned wpo_variant = 0;
@@ -257,6 +261,8 @@ private:
     std::vector<void *> streams_;
 
     void launch_all();
+    void report_effective_arguments();
+    void release() noexcept;
     void launch(const T *left, const T *right, T *out, dsize_t n_left, dsize_t n_right, void *stream);
 };
 

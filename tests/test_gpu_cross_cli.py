@@ -79,7 +79,9 @@ def test_json_arguments_and_properties(tmp_path, oracle):
     assert float(out.strip().splitlines()[1].split(",")[0]) < 1e-5
     header, row = (tmp_path / "t.csv").read_text().strip().splitlines()
     assert header == "Kernel,Kernel_iterations,warps_per_thread_block,shifts_per_thread_right_matrix,right_matrices_per_thread,left_rows_per_iteration"
-    assert row.split(",")[2:] == ["4", "2", "2", "1"]
+    # the tile-selecting integers are exact requests, answered by the nearest compiled tile at or above them, and the
+    # measurement file reports what ran: 2 y shifts -> the 4-shift tile, 2 right matrices -> 4 (one per lane, four lanes)
+    assert row.split(",")[2:] == ["4", "4", "4", "1"]
     got = read_matrices(tmp_path / "o.csv")
     exp = oracle.one_to_many(left, right)
     assert np.abs(got - exp).max() <= 1e-3 * np.abs(exp).max()
@@ -95,6 +97,65 @@ def test_json_arguments_and_properties(tmp_path, oracle):
     assert rc == 0, err
     header, row = (tmp_path / "t2.csv").read_text().strip().splitlines()
     assert header.endswith("warps_per_thread_block,rows_per_thread,distribution_type") and row.endswith("8,4,triangle")
+
+
+def test_tuning_integers_select_tiles(tmp_path, oracle):
+    """shifts_per_thread 4 / 8 in the arguments file run the 4- / 8-shift tiles (reported in the measurement file);
+    without the key the library chooses by itself; results are the same."""
+    rng = np.random.default_rng(45)
+    left = rng.integers(-3, 4, (1, 150, 140)).astype(np.float32)
+    right = rng.integers(-3, 4, (1, 150, 140)).astype(np.float32)
+    lp, rp = write_matrices(tmp_path / "l.csv", left), write_matrices(tmp_path / "r.csv", right)
+    exp = oracle.one_to_one(left[0], right[0])
+    seen = {}
+    for label, kw in [("none", {}), ("four", dict(shifts_per_thread=4)), ("eight", dict(shifts_per_thread=8)), ("three", dict(shifts_per_thread=3)),
+                      ("five", dict(shifts_per_thread=5))]:
+        args = write_args(tmp_path / f"{label}.json", **kw)
+        rc, out, err = run_cross("run", "--args_path", args, "--no_progress", "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / f"{label}_t.csv",
+                                 "--out", tmp_path / f"{label}_o.csv", "nai_shuffle_multirow_both_one_to_one", lp, rp, cwd=tmp_path)
+        assert rc == 0, err
+        header, row = (tmp_path / f"{label}_t.csv").read_text().strip().splitlines()
+        seen[label] = dict(zip(header.split(","), row.split(",")))["shifts_per_thread"]
+        np.testing.assert_array_equal(read_matrices(tmp_path / f"{label}_o.csv")[0], exp[0], err_msg=label)
+    assert seen["four"] == "4" and seen["three"] == "4" and seen["eight"] == "8" and seen["five"] == "8", seen
+    assert seen["none"] in ("4", "8")
+    # n_to_m: matrices per thread pick the lanes-over-matrices tiles
+    left = rng.integers(-3, 4, (8, 30, 30)).astype(np.float32)
+    right = rng.integers(-3, 4, (8, 30, 30)).astype(np.float32)
+    lp, rp = write_matrices(tmp_path / "l8.csv", left), write_matrices(tmp_path / "r8.csv", right)
+    exp = oracle.n_to_m(left, right)
+    for lm, rm in [(1, 1), (4, 4), (2, 3)]:
+        args = write_args(tmp_path / "m.json", left_matrices_per_thread=lm, right_matrices_per_thread=rm)
+        rc, out, err = run_cross("run", "--args_path", args, "--no_progress", "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / "m_t.csv",
+                                 "--out", tmp_path / "m_o.csv", "nai_shuffle_multirow_both_multimat_both_n_to_m", lp, rp, cwd=tmp_path)
+        assert rc == 0, err
+        header, row = (tmp_path / "m_t.csv").read_text().strip().splitlines()
+        props = dict(zip(header.split(","), row.split(",")))
+        assert int(props["left_matrices_per_thread"]) >= lm and int(props["right_matrices_per_thread"]) >= rm, props
+        if (lm, rm) == (1, 1):
+            assert props["left_matrices_per_thread"] == "1" and props["right_matrices_per_thread"] == "1", props
+        if (lm, rm) == (4, 4):
+            assert props["left_matrices_per_thread"] == "4" and props["right_matrices_per_thread"] == "4", props
+        np.testing.assert_array_equal(read_matrices(tmp_path / "m_o.csv"), exp)
+
+
+def test_fft_algorithm_repeated_by_min_time_still_validates(tmp_path, oracle):
+    """An fft_* algorithm measured with a min_time that forces many repetitions: the in-place hadamard and the
+    input-consuming inverse transform are repeated, and the stored / validated result must still be that of one pass."""
+    rng = np.random.default_rng(46)
+    left = rng.random((1, 32, 32), dtype=np.float32)
+    right = rng.random((1, 32, 32), dtype=np.float32)
+    lp, rp = write_matrices(tmp_path / "l.csv", left), write_matrices(tmp_path / "r.csv", right)
+    rc, out, err = run_cross("run", "--validate", "--normalize", "--no_progress", "-b", "Algorithm", "-m", "0.02", "-t", tmp_path / "t.csv",
+                             "--out", tmp_path / "o.csv", "fft_orig_one_to_one", lp, rp, cwd=tmp_path)
+    assert rc == 0, err
+    header, row = (tmp_path / "t.csv").read_text().strip().splitlines()
+    cols = dict(zip(header.split(","), row.split(",")))
+    assert int(cols["Hadamard_iterations"]) > 1 and int(cols["Inverse FFT_iterations"]) > 1, cols
+    exp = oracle.one_to_one(left[0], right[0])
+    assert float(out.strip().splitlines()[1].split(",")[0]) <= 1e-3 * np.abs(exp).max(), out
+    got = read_matrices(tmp_path / "o.csv")
+    assert np.abs(got - exp).max() <= 1e-4 * np.abs(exp).max()
 
 
 def test_common_steps_and_streams(tmp_path, oracle):
@@ -114,3 +175,11 @@ def test_common_steps_and_streams(tmp_path, oracle):
         got = read_matrices(tmp_path / "o.csv")
         exp = oracle.n_to_mn(left, right)
         assert np.abs(got - exp).max() <= 1e-3 * np.abs(exp).max()
+    # without the key: one launch over all left matrices, device-event timing, the default is still reported
+    rc, out, err = run_cross("run", "--validate", "--no_progress", "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / "t1.csv",
+                             "--out", tmp_path / "o1.csv", "nai_shuffle_multirow_both_multimat_right_n_to_mn", lp, rp, cwd=tmp_path)
+    assert rc == 0, err
+    header, row = (tmp_path / "t1.csv").read_text().strip().splitlines()
+    assert header.endswith(",num_cuda_streams") and row.endswith(",8")
+    got = read_matrices(tmp_path / "o1.csv")
+    assert np.abs(got - exp).max() <= 1e-3 * np.abs(exp).max()

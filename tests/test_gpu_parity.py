@@ -312,6 +312,48 @@ def test_every_compiled_specialisation_by_index(oracle):
         assert len(names) >= 9
 
 
+def test_tuning_integers_are_exact_requests(oracle):
+    """The reference's shifts / matrices per thread, when non-zero, pick the nearest compiled tile at or above them
+    (xcorr_last_launch tells which); zero leaves the choice to the launcher. Results do not depend on the tile."""
+    xc = load_package()
+    rng = np.random.default_rng(11)
+    left, right = ints(rng, (130, 150), np.float32), ints(rng, (130, 150), np.float32)
+    exp = oracle.one_to_one(left, right)
+    for asked, want in [(1, 4), (2, 4), (4, 4), (5, 8), (8, 8)]:
+        got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(shifts_per_thread=asked))
+        rec = xc.last_launch()
+        assert rec["y_shifts_per_thread"] == want, (asked, rec)
+        check(got, exp, True, f"grouped shifts_per_thread={asked}")
+    for dtype in (np.float32, np.float64):
+        left, right = ints(rng, (1, 40, 40), dtype), ints(rng, (20, 40, 40), dtype)
+        exp = oracle.one_to_many(left[0], right)
+        for asked in (1, 2, 4):
+            got = xc.run("multimat_right_grouped", left, right, 20, n_left=1, n_right=20, params=xc.make_params(right_matrices_per_thread=asked))
+            rec = xc.last_launch()
+            have = rec["right_matrices_per_thread"] * rec["lanes_right"]
+            assert have == (1 if asked == 1 else 4), (asked, rec)
+            check(got, exp, True, f"right_matrices_per_thread={asked}")
+        left, right = ints(rng, (6, 24, 24), dtype), ints(rng, (9, 24, 24), dtype)
+        exp = oracle.n_to_m(left, right)
+        for lm, rm in [(1, 1), (4, 4), (3, 2), (4, 1)]:
+            got = xc.run("multimat_both_grouped", left, right, 54, n_left=6, n_right=9,
+                         params=xc.make_params(left_matrices_per_thread=lm, right_matrices_per_thread=rm))
+            rec = xc.last_launch()
+            assert rec["right_matrices_per_thread"] * rec["lanes_right"] >= rm and rec["left_matrices_per_thread"] * rec["lanes_left"] >= lm, (lm, rm, rec)
+            if (lm, rm) == (1, 1):
+                assert rec["lanes_right"] == 1 and rec["lanes_left"] == 1, rec
+            check(got, exp, True, f"left/right matrices per thread {lm}/{rm}")
+        # one-output-row families
+        got = xc.run("multimat_both", left, right, 54, n_left=6, n_right=9, params=xc.make_params(left_matrices_per_thread=2, right_matrices_per_thread=2, rows_per_thread=8))
+        rec = xc.last_launch()
+        assert rec["left_matrices_per_thread"] == 2 and rec["right_matrices_per_thread"] == 2, rec
+        check(got, exp, True, "multimat_both 2/2")
+        got = xc.run("multimat_both", left, right, 54, n_left=6, n_right=9, params=xc.make_params(left_matrices_per_thread=1, right_matrices_per_thread=1, rows_per_thread=8))
+        rec = xc.last_launch()
+        assert rec["left_matrices_per_thread"] == 1 and rec["right_matrices_per_thread"] == 1, rec
+        check(got, exp, True, "multimat_both 1/1")
+
+
 def test_launch_record_and_errors(oracle):
     xc = load_package()
     rng = np.random.default_rng(700)
