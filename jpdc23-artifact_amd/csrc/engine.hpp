@@ -398,10 +398,12 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         u_limit = g.nU;
     }
 
-    // right columns with any overlap for this block tile, aligned down to the staging width
+    // right columns with any overlap for this block tile, from the first K-column chunk that has some on: the first
+    // stage then starts with useful chunks for all wavefronts that split it (aligned to the staging width instead,
+    // the first and the last stage of a tile were both partly empty)
     int xr_lo = -(sxb + C::TXB - 1);
     if (xr_lo < 0) xr_lo = 0;
-    xr_lo = (xr_lo / C::KBX) * C::KBX;
+    xr_lo = (xr_lo / K) * K;
     int xr_hi = W - sxb;
     if (xr_hi > W) xr_hi = W;
     // this work item's chunk of those columns: [xr_lo, xr_hi) shrinks to it, and w_hi (= W when the

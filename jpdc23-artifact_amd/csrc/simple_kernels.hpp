@@ -345,9 +345,23 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
 // warp-per-shift kernel (naive_warp_per_shift_shared_mem.cu:160-420, its fastest at 64x64) reaches for with
 // its row slabs. Tasks are dealt so that the wavefronts of a block get output rows far apart (a mix of
 // long and short overlaps on every CU).
-template <typename T, int A, int B, int U>
+// (Indices are split into row and column by multiplication with a rounded-up reciprocal that the host passes in:
+// the integer divisions the compiler would emit for run-time pitches cost about forty instructions each, and the
+// copy into LDS was bound by them.)
+struct PairGeometry {
+    int W, H, pitch_l, pitch_r, tasks_x, total_tasks;
+    unsigned magic_pl, magic_pr, magic_tx; // floor(2^32 / d) + 1 for d = pieces per left row, per right row, tasks per output row
+};
+__device__ __forceinline__ int div_by(int n, int d, unsigned magic) { return d == 1 ? n : (int)__umulhi((unsigned)n, magic); }
+
+// COLS != 0 compiles the kernel for matrices of exactly that many columns: the row pitches of the LDS images are then
+// constants and every LDS read of a round is the round's base address plus an immediate offset (with run-time pitches
+// one address addition per read, two thirds as many instructions again as the FMAs).
+template <typename T, int A, int B, int U, int COLS>
 __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left, const T *__restrict__ right, T *__restrict__ out,
-                                                           int W, int H, int pitch_l, int pitch_r, int tasks_x, int total_tasks) {
+                                                           const PairGeometry geo) {
+    const int W = COLS ? COLS : geo.W, H = geo.H, tasks_x = geo.tasks_x, total_tasks = geo.total_tasks;
+    const int pitch_l = COLS ? COLS + 2 * (B < 16 / (int)sizeof(T) ? 16 / (int)sizeof(T) : B) : geo.pitch_l, pitch_r = COLS ? COLS : geo.pitch_r;
     using vec = typename vec128<T>::type;
     constexpr int VK = 16 / (int)sizeof(T);
     constexpr int PAD = B < VK ? VK : B;          // zero columns on either side of a left row (keeps 128-bit pieces aligned)
@@ -372,7 +386,8 @@ __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__
                 if (p >= total) continue;
                 const bool is_left = p < total_l;
                 const int q = is_left ? p : p - total_l, pp = is_left ? pl : pr;
-                const int row = q / pp - (is_left ? TOP : 0), col = (q % pp) * VK - (is_left ? PAD : 0); // matrix row, first column
+                const int qrow = div_by(q, pp, is_left ? geo.magic_pl : geo.magic_pr);
+                const int row = qrow - (is_left ? TOP : 0), col = (q - qrow * pp) * VK - (is_left ? PAD : 0); // matrix row, first column
                 if (row < 0 || row >= H) continue;
                 const T *src = (is_left ? left : right) + (size_t)row * W + col;
                 if (col >= 0 && col + VK <= W) {
@@ -395,7 +410,8 @@ __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     // task (wave w of block b, round i) = w * gridDim + b + i * gridDim * nw
     for (int t = wave * (int)gridDim.x + (int)blockIdx.x; t < total_tasks; t += (int)gridDim.x * nw) {
-        const int oy0 = (t / tasks_x) * A, ox0 = (t % tasks_x) * B;
+        const int ty = div_by(t, tasks_x, geo.magic_tx);
+        const int oy0 = ty * A, ox0 = (t - ty * tasks_x) * B;
         const int sy0 = oy0 - (H - 1), sx0 = ox0 - (W - 1);
         // right rows / columns that overlap any of the A x B shifts
         int y_lo = -(sy0 + A - 1), y_hi = H - sy0, x_lo = -(sx0 + B - 1), x_hi = W - sx0;
@@ -473,7 +489,7 @@ inline bool pair_fits_lds(unsigned cols, unsigned rows) {
     return pair_in_lds_bytes<T>(cols, rows, 2, 4) <= 160 * 1024;
 }
 
-template <typename T, int A, int U>
+template <typename T, int A, int U, int COLS>
 int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, unsigned rows, size_t bytes, unsigned *grid_out,
                        unsigned *waves_out, hipStream_t stream) {
     constexpr unsigned VK = 16 / sizeof(T), B = PAIR_B, PAD = B < VK ? VK : B;
@@ -482,7 +498,7 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     int dev = 0;
     XCORR_HIP(hipGetDevice(&dev));
     if (bytes > 64 * 1024 && !(dev >= 0 && dev < 64 && attr_set[dev])) {
-        XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, A, B, U>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, A, B, U, COLS>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024));
         if (dev >= 0 && dev < 64) attr_set[dev] = true;
     }
@@ -497,8 +513,10 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     const unsigned waves = total <= 8u * (unsigned)cus ? 8 : 16;
     unsigned grid = (total + waves - 1) / waves;
     if (grid > (unsigned)cus) grid = (unsigned)cus; // one block per CU: every block pays for its own copy of the pair
-    pair_in_lds_kernel<T, A, B, U><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, (int)cols, (int)rows, pitch_l, pitch_r,
-                                                                                    (int)tasks_x, (int)total);
+    auto magic = [](unsigned d) { return (unsigned)((1ull << 32) / d) + 1u; }; // exact for n * d < 2^32, far above any index here
+    const PairGeometry geo = {(int)cols,         (int)rows,          pitch_l,       pitch_r, (int)tasks_x, (int)total,
+                              magic(pitch_l / VK), magic(pitch_r / VK), magic(tasks_x)};
+    pair_in_lds_kernel<T, A, B, U, COLS><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, geo);
     XCORR_HIP(hipGetLastError());
     *grid_out = grid;
     *waves_out = waves;
@@ -518,10 +536,21 @@ int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, u
     const size_t bytes = pair_in_lds_bytes<T>(cols, rows, A, U);
     unsigned grid = 0, waves = 0;
     int rc;
-    if (A == 1)
-        rc = launch_pair_in_lds<T, 1, U>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    // the column counts the reference's benchmarks use are compiled in (multiples of 16 whose pitches need no rounding)
+    if (A == 1 && cols == 64)
+        rc = launch_pair_in_lds<T, 1, U, 64>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else if (A == 1 && cols == 32)
+        rc = launch_pair_in_lds<T, 1, U, 32>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else if (A == 1 && cols == 16)
+        rc = launch_pair_in_lds<T, 1, U, 16>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else if (A == 1)
+        rc = launch_pair_in_lds<T, 1, U, 0>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else if (cols == 64)
+        rc = launch_pair_in_lds<T, 2, U, 64>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+    else if (cols == 96)
+        rc = launch_pair_in_lds<T, 2, U, 96>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
     else
-        rc = launch_pair_in_lds<T, 2, U>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 2, U, 0>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
     if (rc != XCORR_OK) return rc;
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
