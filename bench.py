@@ -73,9 +73,9 @@ def cpu_baseline(oracle, cfg, left, right, budget_s=15.0):
 class Workload:
     """One benchmark configuration resident in HBM: inputs copied once, output buffer allocated once."""
 
-    def __init__(self, xc, workloads, name, family=None, params_json="{}", data="config"):
+    def __init__(self, xc, workloads, name, family=None, params_json="{}", data="config", cfg=None):
         self.xc, self.name = xc, name
-        self.cfg = cfg = dict(workloads.CONFIGS[name], name=name)
+        self.cfg = cfg = dict(cfg if cfg is not None else workloads.CONFIGS[name], name=name)
         self.family = family or cfg["family"]
         self.dtype = np.dtype(cfg["dtype"])
         self.left, self.right = workloads.generate(cfg, integer_valued=data != "config")
@@ -206,6 +206,9 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="C2")
+    ap.add_argument("--shape", default=None, metavar="MODE:N_LEFT:N_RIGHT:SIZE[:DTYPE]",
+                    help="time another shape than the five configurations, e.g. n_to_m:4:8:128:float64 (square matrices, uniform [0,1) values, "
+                         "seed 2023, the mode's grouped family unless --family says otherwise); implies --only")
     ap.add_argument("--family", default=None)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--only", action="store_true", help="time --config alone (the default C2 run also times C1, C3, C4 and C5 and reports them under \"per_config\")")
@@ -229,7 +232,15 @@ def main():
     from jpdc23_artifact_amd import workloads
 
     default_launch = args.family is None and args.params == "{}"
-    w = Workload(xc, workloads, args.config, args.family, args.params, args.data)
+    custom = None
+    if args.shape:
+        mode, n_left, n_right, size, *rest = args.shape.split(":")
+        family = {"one_to_one": "grouped_overlap", "one_to_many": "multimat_right_grouped", "n_to_mn": "multimat_right_grouped",
+                  "n_to_m": "multimat_both_grouped"}[mode]
+        custom = dict(mode=mode, dtype=rest[0] if rest else "float32", rows=int(size), cols=int(size), n_left=int(n_left), n_right=int(n_right),
+                      dist="uniform", seed=2023, family=family)
+        args.config, args.only = args.shape, True
+    w = Workload(xc, workloads, args.config, args.family, args.params, args.data, cfg=custom)
     cfg, dtype, rows, cols, pairs = w.cfg, w.dtype, w.rows, w.cols, w.pairs
 
     if args.calibrate_copy:

@@ -25,8 +25,22 @@
  *     across this boundary;
  *   - a tuning field of xcorr_params set to 0 selects the library's tuned default;
  *   - after a successful launch the geometry actually used is available from
- *     xcorr_last_launch() (reference kernel_args.hpp:9-33, a process-global that
- *     is not thread-safe there either).
+ *     xcorr_last_launch() (reference kernel_args.hpp:9-33, one record per process
+ *     there; here one per host thread, like the error message);
+ *   - `left`, `right` and `out` are ordinary device allocations (hipMalloc /
+ *     xcorr_malloc: coarse-grained memory of the current device). Launches that
+ *     split a reduction add partial sums with the hardware's floating-point
+ *     atomic add (xcorr_last_launch().uses_atomics == 1: the split-row families
+ *     always, the grouped families when the launcher cuts the reduction to fill
+ *     the device). That instruction is only defined on coarse-grained memory -
+ *     on fine-grained, host-mapped or managed allocations it is silently dropped -
+ *     and the order of the additions, hence the last bits of such a result, varies
+ *     from run to run. rows_per_thread >= rows together with column_chunks = 1
+ *     asks a grouped family for the launch without atomics, whose result is the
+ *     same bits every run;
+ *   - host threads may launch side by side (error text, launch record and plan cache
+ *     are per thread); the library keeps per-device facts for up to 64 devices and
+ *     always works on the calling thread's current device.
  */
 #ifndef XCORR_HIP_H
 #define XCORR_HIP_H

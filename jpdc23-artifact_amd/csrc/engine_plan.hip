@@ -10,19 +10,6 @@
 
 namespace xcorr {
 
-static int device_cus() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0)
-            cus = prop.multiProcessorCount;
-        else
-            cus = 256;
-    }
-    return cus;
-}
-
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Relative cost of running a request of the one-output-row families on one of their tiles
@@ -371,20 +358,22 @@ static bool same_shape(const EngineRequest &a, const EngineRequest &b) {
 static int cached_plan(const EngineRequest &rq, EnginePlan &plan) {
     struct Entry {
         bool used;
+        int dev; // plans depend on the device's CU count and occupancy
         EngineRequest rq;
         EnginePlan plan;
     };
     constexpr int N = 8;
     thread_local Entry cache[N] = {};
     thread_local int next = 0;
+    const int dev = current_device();
     for (int i = 0; i < N; ++i)
-        if (cache[i].used && same_shape(cache[i].rq, rq)) {
+        if (cache[i].used && cache[i].dev == dev && same_shape(cache[i].rq, rq)) {
             plan = cache[i].plan;
             return XCORR_OK;
         }
     int rc = plan_engine(rq, plan);
     if (rc != XCORR_OK) return rc;
-    cache[next] = Entry{true, rq, plan};
+    cache[next] = Entry{true, dev, rq, plan};
     next = (next + 1) % N;
     return XCORR_OK;
 }

@@ -64,17 +64,18 @@ hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
 
 template <class C>
 int resident_blocks_engine() {
-    static int blocks = 0;
-    if (blocks == 0) {
+    static int blocks[MAX_DEVICES] = {}; // per device: another device may hold another number
+    const int dev = current_device();
+    if (blocks[dev] == 0) {
         int n = 0;
         if (allow_large_lds<C>() != hipSuccess ||
             hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(&engine_kernel<C>), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
             (void)hipGetLastError();
             n = 1;
         }
-        blocks = n;
+        blocks[dev] = n;
     }
-    return blocks;
+    return blocks[dev];
 }
 
 template <class C>

@@ -504,11 +504,7 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     }
     const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
     const unsigned tasks_x = (Sx + B - 1) / B, total = tasks_x * ((Sy + A - 1) / A);
-    static int cus = 0;
-    if (cus == 0) {
-        hipDeviceProp_t prop;
-        cus = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    }
+    const int cus = device_cus();
     // eight wavefronts per block while that still gives every task a wavefront of its own, else sixteen
     const unsigned waves = total <= 8u * (unsigned)cus ? 8 : 16;
     unsigned grid = (total + waves - 1) / waves;

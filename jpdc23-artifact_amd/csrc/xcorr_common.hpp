@@ -39,14 +39,32 @@ inline int hip_check(hipError_t e, const char *what) {
         if (_rc != XCORR_OK) return _rc;                 \
     } while (0)
 
-// ---- last launch record (process-global, like reference kernel_args.cpp:7-19) ----
+// ---- last launch record (reference kernel_args.cpp:7-19 keeps one per process; here one per host thread, like the
+// error text, so that threads launching side by side do not overwrite each other's record) ----
 inline xcorr_launch_record &last_launch() {
-    static xcorr_launch_record rec;
+    static thread_local xcorr_launch_record rec;
     return rec;
 }
 inline bool &have_last_launch() {
-    static bool have = false;
+    static thread_local bool have = false;
     return have;
+}
+
+// ---- per-device facts that are asked of the runtime once ----
+constexpr int MAX_DEVICES = 64;
+inline int current_device() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return 0;
+    return dev;
+}
+inline int device_cus() {
+    static int cus[MAX_DEVICES] = {};
+    const int dev = current_device();
+    if (cus[dev] == 0) {
+        hipDeviceProp_t prop;
+        cus[dev] = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    }
+    return cus[dev];
 }
 
 // Release limits of the reference build (CMakeLists.txt:16-46).

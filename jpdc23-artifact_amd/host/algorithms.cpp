@@ -359,7 +359,8 @@ template <typename T>
 void gpu_algorithm<T>::launch_all() {
     const dsize_t n = refs_.num_matrices(), total_right = targets_.num_matrices();
     const std::size_t in_area = refs_.matrix_size().area(), out_area = results_.matrix_size().area();
-    if (zero_output_) xcheck(xcorr_memset_async(d_results_, 0, results_.size() * sizeof(T), nullptr));
+    // (the clear is a small fill kernel: shorter than a memset command for the outputs of small instances, and it may be captured)
+    if (zero_output_) xcheck(xcorr_clear_async(d_results_, results_.size() * sizeof(T), nullptr));
     if (def_.per_left_streams) {
         if (zero_output_) xcheck(xcorr_device_sync()); // the clear runs on the default stream
         // one launch per left matrix, left r on stream r mod k (n_to_mn.hpp:553-571, n_to_m.hpp:198-212)
