@@ -21,14 +21,15 @@ from __graft_entry__ import load_oracle, load_package  # noqa: E402
 
 # MI355X published vector peaks (TFLOP/s)
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
-# by the library's copy kernel (figures and commands: profiles/engine_f32_a8b4_one_to_one_1024.md, profiles/engine_other_workloads.md).
+# HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
+# by the library's copy kernel (figures and commands in the profile each entry names). Not measured in this run:
 # Keyed by (workload, kernel of the launch record): a default launch that picks another tile reports null.
 MEASURED_TRAFFIC = {
-    ("C2", "grouped_overlap/f32_a8b4"): (2.232e9 + 0.636e9, "profiles/engine_f32_a8b4_one_to_one_1024.md"),
-    ("C3", "multimat_right_grouped/f32_a8b4_lr8"): (0.0253e9 + 0.143e9, "profiles/engine_other_workloads.md"),
-    ("C4", "multimat_right_grouped/f32_a8b4_lr8"): (0.0114e9 + 0.062e9, "profiles/engine_other_workloads.md"),
-    ("C5", "multimat_both_grouped/f64_a8b4_ll4lr8"): (0.006e9 + 0.108e9, "profiles/engine_other_workloads.md"),
+    ("C1", "grouped_overlap/pair_in_lds_f32_a1"): (0.32e6 + 0.18e6, "profiles/pair_in_lds_one_to_one_64.md"),
+    ("C2", "grouped_overlap/f32_a8b4"): (2.360e9 + 0.703e9, "profiles/engine_f32_a8b4_one_to_one_1024.md"),
+    ("C3", "multimat_right_grouped/f32_a8b4_lr8"): (0.0253e9 + 0.1430e9, "profiles/engine_other_workloads.md"),
+    ("C4", "multimat_right_grouped/f32_a8b4_lr8"): (0.0114e9 + 0.0619e9, "profiles/engine_other_workloads.md"),
+    ("C5", "multimat_both_grouped/f64_a8b4_ll4lr8"): (0.0070e9 + 0.1100e9, "profiles/engine_other_workloads.md"),
 }
 
 
