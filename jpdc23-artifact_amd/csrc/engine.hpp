@@ -61,16 +61,17 @@ struct EngineArgs {
 // overlaps), and the longest work item of a launch is WZ_ times shorter. The partial sums are
 // added through LDS before the tile is written (or atomically added, once per block, when the
 // reduction is also split over work items).
+// SB_: 128-bit pieces a thread loads from global memory before it writes the first of them to LDS when staging a band set.
 // DB_ = 1: two sets of LDS bands. While the wavefronts sweep one, the next stage is copied into the
 // other by the memory pipeline itself (loads that write LDS directly, no registers, no waiting
 // wavefront), and one barrier per stage is enough.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
-          int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0>
+          int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0, int SB_ = 8>
 struct EngineCfg {
     using value_type = T;
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
-    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_;
+    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_, SB = SB_;
     static constexpr int VK = 16 / (int)sizeof(T); // elements per 128-bit LDS access
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
@@ -131,7 +132,7 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
 // is src[band][row0 + row][col0 + col] if band < nbands, row_lo <= row < row_hi and
 // col_lo <= col < col_hi, and zero otherwise (the caller passes ranges that keep the reads
 // inside the matrices). Every thread moves 128-bit pieces; the loads of up to eight pieces are
-// issued back to back before the first LDS write, so their latencies overlap.
+// issued back to back before the first LDS write (C::SB of them), so their latencies overlap.
 template <class C, int NB, int ROWS, int PITCH, int BAND>
 __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride, int W,
                                             int nbands, int row_lo, int row_hi, int row0, int col0, int col_lo, int col_hi, int tid) {
@@ -139,7 +140,7 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
     using vec = typename vec128<T>::type;
     constexpr int VK = C::VK, PP = PITCH / VK, TOTP = NB * ROWS * PP;
     constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
-    constexpr int BATCH = ITER < 8 ? ITER : 8;
+    constexpr int BATCH = ITER < C::SB ? ITER : C::SB;
     static_assert(PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
 #pragma unroll
     for (int it0 = 0; it0 < ITER; it0 += BATCH) {

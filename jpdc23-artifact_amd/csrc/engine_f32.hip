@@ -32,8 +32,9 @@ using Z_88_u16 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 1, 16, 1, 1, 18, 16, 3, 4
 using Z_84_v4u4 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v4u4 = EngineCfg<float, 8, 8, 4, 1, 1, 2, 2, 4, 4, 1, 1, 18, 16, 4, 4>;
 using Z_88_v8u8 = EngineCfg<float, 8, 8, 4, 1, 1, 1, 1, 8, 8, 1, 1, 18, 16, 4, 4>;
-// (168 registers, three wavefronts per SIMD: the eight band offsets per lane spill less, measured 1.6 % faster than at 128)
-using Z_84_u8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 3, 4>;
+// (168 registers, three wavefronts per SIMD: measured 1.6-3 % faster than at 128, where 42 registers spill; with that budget all nine
+// pieces a thread stages per band set are loaded before the first LDS write - last parameter -, another 1 %)
+using Z_84_u8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 36, 16, 3, 4, 0, 12>;
 // lanes over 4 x 8 pairs: 8x8 shifts per wavefront, the least tile-edge work for n_to_m of small matrices (also 168 registers:
 // 3-4 % faster than at 128, and than the 4 x 4 pair tile, on 32x32 and 64x64 matrices)
 using Z_84_v4u8 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 1, 4, 8, 1, 1, 18, 16, 3, 4>;
