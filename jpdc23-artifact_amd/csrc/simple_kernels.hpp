@@ -527,8 +527,7 @@ int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, u
     // one / two y shifts per task: fp32 64x64 6.0 / 6.8, 96x96 17.0 / 14.1, 128x128 46 / 29; fp64 32x32 4.4 / 5.0,
     // 64x64 9.0 / 8.6, 96x96 27 / 19. Eight rows per round instead of four changed nothing.
     constexpr unsigned U = 4;
-    unsigned A = (size_t)cols * rows <= (sizeof(T) == 4 ? 88u * 88u : 40u * 40u) ? 1 : 2;
-    if (pair_in_lds_bytes<T>(cols, rows, A, U) > 160 * 1024) A = 2;
+    const unsigned A = (size_t)cols * rows <= (sizeof(T) == 4 ? 88u * 88u : 40u * 40u) ? 1 : 2;
     const size_t bytes = pair_in_lds_bytes<T>(cols, rows, A, U);
     unsigned grid = 0, waves = 0;
     int rc;
