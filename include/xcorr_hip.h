@@ -88,7 +88,8 @@ extern "C" {
 typedef struct xcorr_params {
     unsigned warps_per_thread_block;         /* <= 32 */
     unsigned shifts_per_thread_block;        /* <= 32, warp-per-overlap family */
-    unsigned rows_per_thread;                /* split-row: max overlap rows per worker (JSON rows_per_thread / rows_per_warp) */
+    unsigned rows_per_thread;                /* split-row: max overlap rows per worker (JSON rows_per_thread / rows_per_warp);
+                                                0 in xcorr_split_row: the library picks the chunk */
     unsigned distribution_type;              /* XCORR_DIST_* */
     unsigned shifts_per_thread;              /* grouped-overlap, <= 8 */
     unsigned left_rows_per_iteration;        /* grouped-overlap <= 8, combined kernels <= 4 */

@@ -264,7 +264,11 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
             if (std::string(a.key) == "num_cuda_streams") num_streams_ = value;
             shown = std::to_string(value);
         }
-        if (a.field) params_.*(a.field) = selects_tile(a.key) && !args.contains(a.key) ? 0u : value;
+        // (the split-row family also takes its chunk of rows from the library unless the file names one: the reference's
+        // default of 10 rows leaves most of the GPU idle on a single small pair)
+        const bool library_default =
+            !args.contains(a.key) && (selects_tile(a.key) || (def.family == Family::split_row && std::string(a.key) == "rows_per_thread"));
+        if (a.field) params_.*(a.field) = library_default ? 0u : value;
         if (a.report) props_.emplace_back(a.key, shown);
     }
     if (def.shared_mem_rows_rule && shared_mem_rows < shifts_per_thread_block) {
@@ -408,6 +412,8 @@ void gpu_algorithm<T>::report_effective_arguments() {
             value = std::to_string(rec.right_matrices_per_thread * (rec.lanes_right ? rec.lanes_right : 1u));
         else if (key == "left_matrices_per_thread")
             value = std::to_string(rec.left_matrices_per_thread * (rec.lanes_left ? rec.lanes_left : 1u));
+        else if (key == "rows_per_thread" && def_.family == Family::split_row)
+            value = std::to_string(rec.rows_per_worker);
     }
 }
 

@@ -97,6 +97,14 @@ def test_json_arguments_and_properties(tmp_path, oracle):
     assert rc == 0, err
     header, row = (tmp_path / "t2.csv").read_text().strip().splitlines()
     assert header.endswith("warps_per_thread_block,rows_per_thread,distribution_type") and row.endswith("8,4,triangle")
+    # without rows_per_thread in the file the library picks the chunk (short ones for a single small pair, not the
+    # reference's 10) and the measurement file reports it
+    args = write_args(tmp_path / "d.json", distribution_type="rectangle")
+    rc, _, err = run_cross("run", "--args_path", args, "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / "t3.csv", "--validate", "--no_progress",
+                           "nai_shuffle_work_distribution_one_to_one", lp, lp, cwd=tmp_path)
+    assert rc == 0, err
+    header, row = (tmp_path / "t3.csv").read_text().strip().splitlines()
+    assert row.endswith("8,3,rectangle"), row
 
 
 def test_tuning_integers_select_tiles(tmp_path, oracle):
