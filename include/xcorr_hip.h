@@ -88,8 +88,8 @@ extern "C" {
 typedef struct xcorr_params {
     unsigned warps_per_thread_block;         /* <= 32 */
     unsigned shifts_per_thread_block;        /* <= 32, warp-per-overlap family */
-    unsigned rows_per_thread;                /* split-row: max overlap rows per worker (JSON rows_per_thread / rows_per_warp);
-                                                0 in xcorr_split_row: the library picks the chunk */
+    unsigned rows_per_thread;                /* split-row contract: max overlap rows per worker (JSON rows_per_thread / rows_per_warp);
+                                                0: the library picks the chunk */
     unsigned distribution_type;              /* XCORR_DIST_* */
     unsigned shifts_per_thread;              /* grouped-overlap, <= 8 */
     unsigned left_rows_per_iteration;        /* grouped-overlap <= 8, combined kernels <= 4 */
@@ -265,13 +265,29 @@ int xcorr_grouped_overlap_f64(const double *left, const double *right, double *o
 
 /* Multi-matrix-right: one left matrix against n_right right matrices, each lane
  * reuses a left value for p->right_matrices_per_thread right matrices.
- * Replaces run_ccn_shuffle_multimat_right (kernels.cuh:87-97) when
- * p->rows_per_thread == 0 and run_ccn_shuffle_multimat_right_work_distribution<DIST>
- * (kernels.cuh:130-142; caller zeroes `out`) otherwise. Result i = left x right i. */
+ * Replaces run_ccn_shuffle_multimat_right_work_distribution<DIST> (kernels.cuh:130-142;
+ * THE CALLER ZEROES `out`) when p->rows_per_thread > 0 or p->distribution_type is
+ * rectangle or triangle (rows_per_thread 0 then leaves the chunk to the library), and
+ * run_ccn_shuffle_multimat_right (kernels.cuh:87-97; `out` need not be zeroed)
+ * otherwise. Result i = left x right i. */
 int xcorr_multimat_right_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                              unsigned n_right, const xcorr_params *p, void *stream);
 int xcorr_multimat_right_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                              unsigned n_right, const xcorr_params *p, void *stream);
+
+/* Multi-matrix-right over n_left groups in one launch: left l against the right matrices
+ * [l*n_right, (l+1)*n_right) (the de-interleaved order of n_to_mn.hpp:165-172), result
+ * index = right index; the same results as n_left calls of xcorr_multimat_right on the
+ * consecutive groups, with the same meaning of p (p->rows_per_thread > 0: caller zeroes
+ * `out`). The reference has no such launcher: its host issues one launch per left
+ * matrix on num_cuda_streams streams (n_to_mn.hpp:228-300); on this device the launch
+ * overhead of that loop dominates small matrices. */
+int xcorr_multimat_right_groups_f32(const float *left, const float *right, float *out, unsigned cols,
+                                    unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                    void *stream);
+int xcorr_multimat_right_groups_f64(const double *left, const double *right, double *out, unsigned cols,
+                                    unsigned rows, unsigned n_left, unsigned n_right, const xcorr_params *p,
+                                    void *stream);
 
 /* Multi-matrix-right x grouped-overlap.
  * Replaces run_ccn_shuffle_one_to_many_multirow_both_multimat_right (kernels.cuh:221-234).

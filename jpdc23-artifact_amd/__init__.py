@@ -276,6 +276,7 @@ FAMILIES = {
     "split_row": ("xcorr_split_row", "pair", True),
     "grouped_overlap": ("xcorr_grouped_overlap", "pair", False),
     "multimat_right": ("xcorr_multimat_right", "right", None),
+    "multimat_right_groups": ("xcorr_multimat_right_groups", "both", None),
     "multimat_right_grouped": ("xcorr_multimat_right_grouped", "both", False),
     "multimat_both": ("xcorr_multimat_both", "both", True),
     "multimat_both_grouped": ("xcorr_multimat_both_grouped", "both", False),
@@ -314,8 +315,8 @@ def needs_zeroed_output(family, params):
         return zero
     if family == "warp_per_overlap":
         return params is not None and params.warp_per_overlap_variant == 2
-    if family == "multimat_right":
-        return params is not None and params.rows_per_thread > 0
+    if family in ("multimat_right", "multimat_right_groups"):
+        return params is not None and (params.rows_per_thread > 0 or params.distribution_type in (2, 3))
     if family == "warp_per_overlap_lds":
         return params is not None and params.column_group_per_block != 0
     return False

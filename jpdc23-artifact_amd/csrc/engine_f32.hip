@@ -17,6 +17,11 @@ namespace xcorr {
 using R_1x1 = EngineCfg<float, 1, 8, 4, 1, 1, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_1x4 = EngineCfg<float, 1, 8, 4, 1, 4, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
 using R_2x2 = EngineCfg<float, 1, 8, 4, 2, 2, 8, 8, 1, 1, 2, 2, 8, 32, 4>;
+// the same with 32 x 8 shifts per wavefront and two wavefronts per block (32 x 16 shifts), for matrices so small that
+// the tiles above mostly cover shifts that do not exist
+using N_1x1 = EngineCfg<float, 1, 4, 4, 1, 1, 8, 8, 1, 1, 1, 2, 8, 16, 4>;
+using N_1x4 = EngineCfg<float, 1, 4, 4, 1, 4, 8, 8, 1, 1, 1, 2, 8, 16, 4>;
+using N_2x2 = EngineCfg<float, 1, 4, 4, 2, 2, 8, 8, 1, 1, 1, 2, 8, 16, 4>;
 // grouped tiles: four wavefronts share one tile and its bands and take every fourth chunk of columns of
 // a stage (WZ = 4). Lanes over shifts only ...
 using Z_84 = EngineCfg<float, 8, 4, 4, 1, 1, 8, 8, 1, 1, 1, 1, 36, 32, 4, 4>;
@@ -62,6 +67,9 @@ static const EngineSpec specs[] = {
     make_spec<Z_84_v4u8>("f32_a8b4_ll4lr8", 0.78, 0.973),
     make_spec<Z_44_u4>("f32_a4b4_lr4", 0.86, 2.5),
     make_spec<Z_44_u8>("f32_a4b4_lr8", 0.87, 2.5),
+    make_spec<N_1x1>("f32_a1b4"),
+    make_spec<N_1x4>("f32_a1b4_r4"),
+    make_spec<N_2x2>("f32_a1b4_l2r2"),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {

@@ -10,6 +10,9 @@ namespace xcorr {
 // one output row per lane, 2x2 wavefronts over the shifts
 using R_1x1 = EngineCfg<double, 1, 8, 2, 1, 1, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
 using R_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 2, 2, 8, 16, 4>;
+// the same with 32 x 8 shifts per wavefront and two wavefronts per block, for small matrices
+using N_1x1 = EngineCfg<double, 1, 4, 2, 1, 1, 8, 8, 1, 1, 1, 2, 8, 8, 4>;
+using N_2x2 = EngineCfg<double, 1, 4, 2, 2, 2, 8, 8, 1, 1, 1, 2, 8, 8, 4>;
 // grouped tiles: four wavefronts share one tile and its bands and take every fourth chunk of columns of a stage
 using Z_88 = EngineCfg<double, 8, 8, 2, 1, 1, 8, 8, 1, 1, 1, 1, 36, 16, 2, 4>;
 using Z_44 = EngineCfg<double, 4, 4, 2, 1, 1, 8, 8, 1, 1, 1, 1, 20, 16, 4, 4>;
@@ -44,6 +47,8 @@ static const EngineSpec specs[] = {
     make_spec<D_84_v4u8>("f64_a8b4_ll4lr8", 0.799, 0.0),
     make_spec<Z_44_u4>("f64_a4b4_lr4", 0.82, 1.0),
     make_spec<Z_44_u8>("f64_a4b4_lr8", 0.85, 1.0),
+    make_spec<N_1x1>("f64_a1b4"),
+    make_spec<N_2x2>("f64_a1b4_l2r2_narrow"),
 };
 
 const EngineSpec *engine_specs_f64(int *count) {

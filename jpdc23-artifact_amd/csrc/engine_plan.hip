@@ -18,8 +18,9 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 //     own tile, but the wavefronts of a block wait for each other after every staged band, so both
 //     the wavefront tile and the block tile count;
 //   * lanes idling over matrices that do not exist;
-//   * issue slots lost to LDS reads (a read plus the wait that guards it displace about nine fp32
-//     FMA slots, half as many fp64 ones);
+//   * issue slots lost to LDS reads (a read plus the wait that guards it displace about four fp32
+//     FMA slots, half as many fp64 ones: with that weight the tiles of 32 x shifts per wavefront win up
+//     to 256x256 matrices and the ones of 64 from 512x512 on, as measured);
 //   * several matrices per lane: the register ring of right rows grows, some spills.
 static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     double waste_x = std::sqrt((double)(rq.W + s.TXW()) * (rq.W + s.TXB())) / rq.W;
@@ -31,7 +32,7 @@ static double spec_cost(const EngineSpec &s, const EngineRequest &rq) {
     int vk = 16 / s.elem_bytes;
     double reads = s.NV * ceil_div(s.B + s.K - 1, vk) + s.NU * (s.K / vk);
     double fmas = (double)s.NV * s.NU * s.A * s.B * s.K;
-    cost *= 1.0 + (s.elem_bytes == 4 ? 9.0 : 4.5) * reads / fmas;
+    cost *= 1.0 + (s.elem_bytes == 4 ? 4.0 : 2.0) * reads / fmas;
     if (s.NV * s.NU > 1) cost *= 1.15;
     return cost;
 }
@@ -81,7 +82,7 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
     plan.spec = &s;
     plan.x_chunks = 1;
     plan.x_chunk_cols = rq.W;
-    if (xc > 1 && rq.may_split && !rq.caller_zeroes) {
+    if (xc > 1 && (rq.may_split || rq.caller_zeroes)) {
         const int granule = s.K * s.WZ;
         const int cw = ceil_div(ceil_div(rq.W, xc), granule) * granule;
         plan.x_chunks = ceil_div(rq.W, cw);
@@ -273,52 +274,49 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         return fail(XCORR_ERR_UNSUPPORTED, "%s: no compiled specialisation matches x_shifts_per_thread=%u lanes_x=%u lanes_y=%u",
                     rq.family, rq.x_shifts, rq.lanes_x, rq.lanes_y);
     int rc = (int)rq.rows_per_worker;
-    if (!rq.caller_zeroes && rc <= 0 && rq.may_split) {
-        // Few tiles, or long ones: cut the reduction over left rows into chunks of whole groups until
-        // the launch has about 128 work items per CU; items shorter than 20 rows only pay for tiny
-        // problems that would otherwise leave CUs without work.
+    const bool split_by_default = rq.caller_zeroes ? rq.dist != XCORR_DIST_NONE : rq.may_split;
+    if (rc <= 0 && split_by_default) {
+        // No chunk size from the caller: the chunk with the lowest relative cost
+        //     (1 + 1300 / (chunk rows x columns)) x (1 + 6.7 x CUs / work items).
+        // The first factor is what a work item pays around its sweep (ring start-up, atomic adds of its tile), the second
+        // how badly few items balance over the device. Fitted to measured split-row, multimat-right and multimat-both
+        // launches of 64x64 ... 512x512 fp32 matrices, 1 ... 1024 pairs (it picks 3-5 rows for a single pair up to 96x96,
+        // 8-16 rows around 128x128 ... 512x512, and whole matrices when the pairs alone fill the device).
         EnginePlan whole;
         if (int e = shape_plan(*best, rq, 0, 1, whole)) return e;
-        const long tiles = whole.total_items;
-        const int G = best->A + 1;
-        const int rc_most = 4 * best->RL;
-        if (tiles < 48L * device_cus() || rq.H > rc_most) {
-            const long target = 128L * device_cus();
-            const long per_tile_column = (long)whole.ntx * whole.nvg * whole.nug;
-            const int k_normal = ceil_div(20, G), k_tiny = ceil_div(9, G);
-            const int k_min = per_tile_column * count_chunks(*best, rq.H, whole.nty, k_normal * G, nullptr) < 2L * device_cus() ? k_tiny : k_normal;
-            int k = (rq.H < rc_most ? rq.H : rc_most) / G;
-            for (; k >= k_min; --k) {
-                rc = k * G;
-                if (per_tile_column * count_chunks(*best, rq.H, whole.nty, rc, nullptr) >= target) break;
-            }
-            if (rc <= 0) rc = rq.H;
-        }
-    }
-    if (rq.caller_zeroes && rc <= 0 && rq.dist != XCORR_DIST_NONE) {
-        // split-row contract without a chunk size from the caller: the longest chunk of 8, 4, 2 staged bands that
-        // still gives every CU eight work items, else one band (n-to-m 16 x 32 of 64x64 fp64: 1.30 -> 0.76 ms
-        // against one band; a single pair of small matrices keeps the short chunks it needs to fill the GPU)
-        rc = best->RL;
-        for (int k = 8; k > 1; k /= 2) {
-            EnginePlan longer;
-            if (int e = shape_plan(*best, rq, k * best->RL, 1, longer)) return e;
-            if (longer.total_items >= 8L * device_cus()) {
-                rc = k * best->RL;
-                break;
+        const double per_tile_column = (double)whole.ntx * whole.nvg * whole.nug;
+        auto chunk_cost = [&](int c) {
+            const double items = per_tile_column * count_chunks(*best, rq.H, whole.nty, c, nullptr);
+            return (1.0 + 1300.0 / ((double)c * rq.W)) * (1.0 + 6.7 * device_cus() / items);
+        };
+        const int candidates[] = {3, 5, 8, 16, 32, 64, rq.H};
+        double best_chunk_cost = 0;
+        for (int c : candidates) {
+            if (c > rq.H) continue;
+            const double cost = chunk_cost(c);
+            if (rc <= 0 || cost < best_chunk_cost) {
+                rc = c;
+                best_chunk_cost = cost;
             }
         }
-        if (rc == best->RL) {
-            // fewer than two work items per CU even with one band per chunk: shorter chunks (measured on single fp32
-            // pairs, clear included: 32x32 11.8 -> 9.3 us and 64x64 20.2 -> 15.9 us with 3 rows, 96x96 31.1 -> 28.0 us
-            // with 5; from 128x128 on one band is best)
-            EnginePlan one_band;
-            if (int e = shape_plan(*best, rq, rc, 1, one_band)) return e;
-            if (one_band.total_items < 2L * device_cus()) rc = rq.H <= 64 ? 3 : 5;
-            if (rc > best->RL) rc = best->RL;
+        // A launcher whose contract is a plain store (no zeroed output, the same bits every run, the summation order of
+        // one pass over the rows) and whose whole tiles already give every CU two work items only gives that up for a
+        // predicted gain of 1.4 x or more.
+        if (!rq.caller_zeroes && whole.total_items >= 2L * device_cus() && best_chunk_cost > 0.7 * chunk_cost(rq.H)) rc = rq.H;
+    }
+    int xc = (int)rq.column_chunks;
+    if (xc == 0 && rq.caller_zeroes && rq.dist == XCORR_DIST_NONE) {
+        // The split-row contract (zeroed output, atomic adds) with the rows explicitly left whole: when that gives the
+        // device less than two work items per CU the reduction over right columns is cut instead, into chunks of at
+        // least 16 columns.
+        EnginePlan whole;
+        if (int e = shape_plan(*best, rq, rc, 1, whole)) return e;
+        if (whole.total_items < 2L * device_cus()) {
+            xc = ceil_div(2 * device_cus(), whole.total_items);
+            if (xc > rq.W / 16) xc = rq.W / 16;
         }
     }
-    return shape_plan(*best, rq, rc, 1, plan);
+    return shape_plan(*best, rq, rc, xc > 1 ? xc : 1, plan);
 }
 
 template <typename T>

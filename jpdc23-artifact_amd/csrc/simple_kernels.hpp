@@ -181,7 +181,9 @@ __device__ __forceinline__ WpoWork wpo_distribute(unsigned worker, unsigned max_
 }
 
 // VARIANT 0: lanes stride the flattened overlap; 1: row loop, lanes stride the columns;
-// 2: as 0 but the rows of a shift are split over workers (DIST) and added atomically.
+// 2: the rows of a shift are split over workers (DIST) and added atomically (the reference's kernel strides the
+// flattened part like 0, naive_warp_per_shift.cu:160-175; here the row loop of 1, which is faster and whose
+// summation order is free anyway once parts are added atomically).
 template <typename T, int VARIANT, int DIST>
 __global__ __launch_bounds__(1024) void warp_per_overlap_kernel(const T *__restrict__ left, const T *__restrict__ right,
                                                                  T *__restrict__ out, int W, int H, unsigned max_rows) {
@@ -210,7 +212,7 @@ __global__ __launch_bounds__(1024) void warp_per_overlap_kernel(const T *__restr
     }
     const int ow = xr_hi - xr_lo, oh = yr_hi - yr_lo;
     T sum = T(0);
-    if (VARIANT == 1) {
+    if (VARIANT != 0) {
         // columns outer (one pass up to 64 columns), rows inner and unrolled eight times with
         // independent partial sums: sixteen loads are in flight per lane instead of two, which is
         // what a wavefront that owns a single short reduction needs to hide the cache latency
@@ -294,7 +296,10 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
     const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
     dim3 block(64, spb);
     unsigned grid_y = Sy;
-    unsigned max_rows = p.rows_per_thread ? p.rows_per_thread : 3; // reference default rows_per_warp, one_to_one.hpp:458
+    // rows per worker of the work-distribution variant. The reference's default is 3 (rows_per_warp, one_to_one.hpp:458);
+    // here 0 keeps every shift whole: measured on 16x16 ... 256x256 pairs, any split was slower than none (a worker's
+    // wavefront-wide sum and atomic add cost more than the few rows it saves)
+    unsigned max_rows = p.rows_per_thread ? p.rows_per_thread : rows;
     unsigned dist = p.distribution_type == XCORR_DIST_DEFAULT ? XCORR_DIST_RECTANGLE : p.distribution_type;
     const int variant = (int)p.warp_per_overlap_variant;
     if (variant == 2) {
@@ -663,6 +668,7 @@ int run_warp_per_overlap_lds(const T *left, const T *right, T *out, unsigned col
         return fail(XCORR_ERR_INVALID_ARGUMENT, "Too many shifts per block: %u (max 32)", p.shifts_per_thread_block);
     unsigned nr = p.right_matrices_per_block ? p.right_matrices_per_block : 1;
     if (nr > 8) return fail(XCORR_ERR_INVALID_ARGUMENT, "Invalid number of right matrices per block: %u [1-8]", nr);
+    if (nr > n_right) nr = n_right; // no bands and FMAs for matrices that do not exist
     unsigned nw = p.shifts_per_thread_block ? p.shifts_per_thread_block : 16;
     if (nw > 16) nw = 16; // a block holds at most 16 wavefronts of 64 lanes
     unsigned sr = p.shared_mem_rows ? p.shared_mem_rows : nw;

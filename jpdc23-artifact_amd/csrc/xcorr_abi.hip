@@ -232,8 +232,11 @@ int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     EngineRequest rq = base_request("shuffle", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = 1;
     rq.left_mats = rq.right_mats = 1;
-    rq.dist = XCORR_DIST_NONE;
-    rq.may_split = false;
+    // The reference's launcher never splits the reduction. Here the planner may (clearing the output itself and adding
+    // partial sums atomically) when the launch would otherwise leave most of the device idle; distribution_type "none"
+    // asks for the unsplit launch.
+    rq.may_split = p.distribution_type != XCORR_DIST_NONE;
+    rq.dist = rq.may_split ? XCORR_DIST_DEFAULT : XCORR_DIST_NONE;
     return run_engine(rq, as_stream(stream));
 }
 
@@ -282,25 +285,27 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
 }
 
 template <typename T>
-int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_right,
+int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left, unsigned n_right,
                         const xcorr_params *pp, void *stream) {
     const xcorr_params &p = params_or_default(pp);
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
-    if ((rc = check_counts(1, n_right, false))) return rc;
+    if ((rc = check_counts(n_left, n_right, n_left > 1))) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
-    EngineRequest rq = base_request("multimat_right", sizeof(T), left, right, out, cols, rows, 1, n_right, p);
+    EngineRequest rq = base_request("multimat_right", sizeof(T), left, right, out, cols, rows, n_left, n_left * n_right, p);
+    rq.group_m = n_left > 1 ? (int)n_right : 0; // left l against its own group of n_right right matrices
     rq.y_shifts = 1;
     rq.left_mats = 1;
     rq.right_mats = p.right_matrices_per_thread;
-    if (p.rows_per_thread > 0) { // the work-distribution launcher
+    if (p.rows_per_thread > 0 || p.distribution_type == XCORR_DIST_RECTANGLE || p.distribution_type == XCORR_DIST_TRIANGLE) {
+        // the work-distribution launcher (rows_per_thread 0 with a distribution: the planner picks the chunk)
         rq.rows_per_worker = p.rows_per_thread;
         rq.caller_zeroes = true;
-    } else {
-        rq.dist = XCORR_DIST_NONE;
-        rq.may_split = false;
+    } else { // the plain launcher: split only by the planner's own choice, never with distribution_type "none"
+        rq.may_split = p.distribution_type != XCORR_DIST_NONE;
+        rq.dist = rq.may_split ? XCORR_DIST_DEFAULT : XCORR_DIST_NONE;
     }
     return run_engine(rq, as_stream(stream));
 }
@@ -428,11 +433,11 @@ XCORR_PAIR_ENTRY(xcorr_grouped_overlap, grouped_impl)
 
 int xcorr_multimat_right_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                              unsigned n_right, const xcorr_params *p, void *stream) {
-    return multimat_right_impl<float>(left, right, out, cols, rows, n_right, p, stream);
+    return multimat_right_impl<float>(left, right, out, cols, rows, 1, n_right, p, stream);
 }
 int xcorr_multimat_right_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                              unsigned n_right, const xcorr_params *p, void *stream) {
-    return multimat_right_impl<double>(left, right, out, cols, rows, n_right, p, stream);
+    return multimat_right_impl<double>(left, right, out, cols, rows, 1, n_right, p, stream);
 }
 
 #define XCORR_NM_ENTRY(NAME, IMPL)                                                                                \
@@ -445,6 +450,7 @@ int xcorr_multimat_right_f64(const double *left, const double *right, double *ou
         return IMPL<double>(left, right, out, cols, rows, n_left, n_right, p, stream);                            \
     }
 
+XCORR_NM_ENTRY(xcorr_multimat_right_groups, multimat_right_impl)
 XCORR_NM_ENTRY(xcorr_multimat_right_grouped, multimat_right_grouped_impl)
 XCORR_NM_ENTRY(xcorr_multimat_both, multimat_both_impl)
 XCORR_NM_ENTRY(xcorr_multimat_both_grouped, multimat_both_grouped_impl)

@@ -71,7 +71,9 @@ std::vector<algorithm_def> build_defs() {
     mmr_wd_streams.push_back(streams());
     {
         auto &a = add("nai_shuffle_multimat_right_work_distribution_n_to_mn", Mode::n_to_mn, Family::multimat_right, mmr_wd_streams);
-        a.zero_output = a.per_left_streams = a.deinterleave = true;
+        // one launch over all left matrices unless the arguments file holds num_cuda_streams (then one launch per left
+        // matrix on that many streams like the reference, n_to_mn.hpp:286-300)
+        a.zero_output = a.per_left_streams_if_asked = a.deinterleave = true;
     }
     {
         auto &a = add("nai_shuffle_multimat_right_work_distribution_n_to_m", Mode::n_to_m, Family::multimat_right, mmr_wd_streams);
@@ -174,6 +176,7 @@ struct entry<float> {
     static constexpr auto split_row = xcorr_split_row_f32;
     static constexpr auto grouped_overlap = xcorr_grouped_overlap_f32;
     static constexpr auto multimat_right = xcorr_multimat_right_f32;
+    static constexpr auto multimat_right_groups = xcorr_multimat_right_groups_f32;
     static constexpr auto multimat_right_grouped = xcorr_multimat_right_grouped_f32;
     static constexpr auto multimat_both = xcorr_multimat_both_f32;
     static constexpr auto multimat_both_grouped = xcorr_multimat_both_grouped_f32;
@@ -188,6 +191,7 @@ struct entry<double> {
     static constexpr auto split_row = xcorr_split_row_f64;
     static constexpr auto grouped_overlap = xcorr_grouped_overlap_f64;
     static constexpr auto multimat_right = xcorr_multimat_right_f64;
+    static constexpr auto multimat_right_groups = xcorr_multimat_right_groups_f64;
     static constexpr auto multimat_right_grouped = xcorr_multimat_right_grouped_f64;
     static constexpr auto multimat_both = xcorr_multimat_both_f64;
     static constexpr auto multimat_both_grouped = xcorr_multimat_both_grouped_f64;
@@ -264,10 +268,11 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
             if (std::string(a.key) == "num_cuda_streams") num_streams_ = value;
             shown = std::to_string(value);
         }
-        // (the split-row family also takes its chunk of rows from the library unless the file names one: the reference's
-        // default of 10 rows leaves most of the GPU idle on a single small pair)
-        const bool library_default =
-            !args.contains(a.key) && (selects_tile(a.key) || (def.family == Family::split_row && std::string(a.key) == "rows_per_thread"));
+        // (the split-row launchers of the sliding-window engine also take their chunk of rows from the library unless the file
+        // names one: the reference's default of 10 rows leaves most of the GPU idle on small inputs and cuts large ones too short)
+        const bool engine_split_row = def.family == Family::split_row || def.family == Family::multimat_right || def.family == Family::multimat_both;
+        const bool library_default = !args.contains(a.key) && (selects_tile(a.key) || (engine_split_row && std::string(a.key) == "rows_per_thread") ||
+                                                               (def.family == Family::warp_per_overlap && std::string(a.key) == "rows_per_warp"));
         if (a.field) params_.*(a.field) = library_default ? 0u : value;
         if (a.report) props_.emplace_back(a.key, shown);
     }
@@ -348,7 +353,12 @@ void gpu_algorithm<T>::launch(const T *left, const T *right, T *out, dsize_t n_l
     case Family::shuffle: xcheck(E::shuffle(left, right, out, cols, rows, &params_, stream)); break;
     case Family::split_row: xcheck(E::split_row(left, right, out, cols, rows, &params_, stream)); break;
     case Family::grouped_overlap: xcheck(E::grouped_overlap(left, right, out, cols, rows, &params_, stream)); break;
-    case Family::multimat_right: xcheck(E::multimat_right(left, right, out, cols, rows, n_right, &params_, stream)); break;
+    case Family::multimat_right:
+        if (n_left > 1)
+            xcheck(E::multimat_right_groups(left, right, out, cols, rows, n_left, n_right, &params_, stream));
+        else
+            xcheck(E::multimat_right(left, right, out, cols, rows, n_right, &params_, stream));
+        break;
     case Family::multimat_right_grouped:
         xcheck(E::multimat_right_grouped(left, right, out, cols, rows, n_left, n_right, &params_, stream));
         break;
@@ -412,7 +422,9 @@ void gpu_algorithm<T>::report_effective_arguments() {
             value = std::to_string(rec.right_matrices_per_thread * (rec.lanes_right ? rec.lanes_right : 1u));
         else if (key == "left_matrices_per_thread")
             value = std::to_string(rec.left_matrices_per_thread * (rec.lanes_left ? rec.lanes_left : 1u));
-        else if (key == "rows_per_thread" && def_.family == Family::split_row)
+        else if (key == "rows_per_warp" && def_.family == Family::warp_per_overlap)
+            value = std::to_string(rec.rows_per_worker);
+        else if (key == "rows_per_thread" && (def_.family == Family::split_row || def_.family == Family::multimat_right || def_.family == Family::multimat_both))
             value = std::to_string(rec.rows_per_worker);
     }
 }

@@ -55,7 +55,12 @@ ONE_TO_ONE_CASES = [
     ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="triangle", rows_per_thread=5)),
     ("shuffle", {}),
     ("shuffle", dict(warps_per_thread_block=4)),
+    ("shuffle", dict(distribution_type="none")),
+    ("split_row", {}),
     ("split_row", dict(distribution_type="none")),
+    ("split_row", dict(distribution_type="none", column_chunks=3)),
+    ("split_row", dict(distribution_type="triangle", rows_per_thread=6, column_chunks=2)),
+    ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution")),
     ("split_row", dict(distribution_type="rectangle", rows_per_thread=10)),
     ("split_row", dict(distribution_type="triangle", rows_per_thread=4)),
     ("split_row", dict(distribution_type="triangle", rows_per_thread=1)),
@@ -150,6 +155,9 @@ ONE_TO_MANY_CASES = [
     ("multimat_right", dict(right_matrices_per_thread=8, warps_per_thread_block=4)),
     ("multimat_right", dict(right_matrices_per_thread=2, rows_per_thread=10, distribution_type="rectangle")),
     ("multimat_right", dict(right_matrices_per_thread=4, rows_per_thread=3, distribution_type="triangle")),
+    ("multimat_right", dict(distribution_type="none")),
+    ("multimat_right", dict(distribution_type="triangle")),
+    ("multimat_right", dict(rows_per_thread=1, distribution_type="none")),
     ("multimat_right_grouped", {}),
     ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=4, right_matrices_per_thread=4, left_rows_per_iteration=4)),
     ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=2, right_matrices_per_thread=2, rows_per_thread=16)),
@@ -225,6 +233,27 @@ def test_n_to_mn_one_launch(oracle, dtype, kw):
         got_dev = xc.run("multimat_right_grouped", left, right_dev, n * m, n_left=n, n_right=m, params=xc.make_params(**kw))
         got_file = np.stack([got_dev[slot[i]] for i in range(n * m)])
         check(got_file, exp_file, True, f"n_to_mn {n}x{m} {shape}")
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+@pytest.mark.parametrize("kw", [{}, dict(distribution_type="none"), dict(right_matrices_per_thread=4, distribution_type="rectangle"),
+                                dict(right_matrices_per_thread=2, rows_per_thread=5, distribution_type="triangle"),
+                                dict(rows_per_thread=1, distribution_type="none")], ids=lambda v: str(v).replace(" ", ""))
+def test_multimat_right_groups(oracle, dtype, kw):
+    """xcorr_multimat_right_groups: the one-output-row family over n_left groups in one launch gives what n_left calls of
+    xcorr_multimat_right on the consecutive groups give (the loop of the reference's host, n_to_mn.hpp:286-300)."""
+    xc = load_package()
+    rng = np.random.default_rng(410)
+    for n, m, shape in [(2, 3, (8, 8)), (3, 5, (20, 13)), (8, 4, (32, 32)), (5, 1, (17, 40))]:
+        say("multimat_right_groups", kw, np.dtype(dtype).name, n, m, shape)
+        left = ints(rng, (n,) + shape, dtype)
+        right = ints(rng, (n * m,) + shape, dtype)
+        exp = np.concatenate([oracle.one_to_many(left[l:l + 1], right[l * m:(l + 1) * m]) for l in range(n)])
+        got = xc.run("multimat_right_groups", left, right, n * m, n_left=n, n_right=m, params=xc.make_params(**kw))
+        check(got, exp, True, f"groups {n}x{m} {shape}")
+        one_by_one = np.concatenate([xc.run("multimat_right", left[l:l + 1], right[l * m:(l + 1) * m], m, n_left=1, n_right=m,
+                                            params=xc.make_params(**kw)) for l in range(n)])
+        np.testing.assert_array_equal(got, one_by_one)
 
 
 N_TO_M_CASES = [
