@@ -31,13 +31,14 @@
  *     xcorr_malloc: coarse-grained memory of the current device). Launches that
  *     split a reduction add partial sums with the hardware's floating-point
  *     atomic add (xcorr_last_launch().uses_atomics == 1: the split-row families
- *     always, the grouped families when the launcher cuts the reduction to fill
- *     the device). That instruction is only defined on coarse-grained memory -
+ *     always; the grouped families, xcorr_shuffle and the plain xcorr_multimat_right
+ *     when the launcher cuts the reduction to fill the device, clearing `out` itself). That instruction is only defined on coarse-grained memory -
  *     on fine-grained, host-mapped or managed allocations it is silently dropped -
  *     and the order of the additions, hence the last bits of such a result, varies
  *     from run to run. rows_per_thread >= rows together with column_chunks = 1
- *     asks a grouped family for the launch without atomics, whose result is the
- *     same bits every run;
+ *     asks a grouped family for the launch without atomics, distribution_type =
+ *     XCORR_DIST_NONE asks xcorr_shuffle / the plain xcorr_multimat_right for it;
+ *     its result is the same bits every run;
  *   - host threads may launch side by side (error text, launch record and plan cache
  *     are per thread); the library keeps per-device facts for up to 64 devices and
  *     always works on the calling thread's current device.
@@ -109,7 +110,7 @@ typedef struct xcorr_params {
     unsigned strided_load;                   /* load pattern of the reference's staging; no effect here */
     unsigned column_group_per_block;         /* 1: one block per group of 64 columns, sums added atomically (caller zeroes `out`) */
     unsigned block_size;                     /* block-per-overlap: threads per block, 0 = 128, <= 1024 */
-    unsigned column_chunks;                  /* grouped families: cut the reduction over right columns into this many chunks
+    unsigned column_chunks;                  /* engine families: cut the reduction over right columns into this many chunks
                                                 (atomic adds, like rows_per_thread for rows); 0 = planner decides, no counterpart in the reference */
     unsigned whole_pair_in_lds;              /* grouped-overlap, one small pair: 0 = the launcher decides, 1 = always run the kernel that
                                                 keeps both matrices in LDS (an error if they do not fit), 2 = never; no counterpart
