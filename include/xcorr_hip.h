@@ -203,6 +203,14 @@ int xcorr_overlap_wise_f32(const float *left, const float *right, float *out, un
                            unsigned n_left, unsigned batch, void *stream);
 int xcorr_overlap_wise_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                            unsigned n_left, unsigned batch, void *stream);
+/* The same kernel over all pairs in one launch: every right matrix with every left matrix,
+ * result index = left * n_right + right (the n_to_m mode). The reference's host reaches
+ * that with one launch per left matrix on num_cuda_streams streams (n_to_m.hpp:198-212);
+ * it has no such launcher. */
+int xcorr_overlap_wise_all_pairs_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                     unsigned n_left, unsigned n_right, void *stream);
+int xcorr_overlap_wise_all_pairs_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                     unsigned n_left, unsigned n_right, void *stream);
 
 /* Warp-per-overlap: one wavefront per shift, lanes stride the overlap, DPP reduction.
  * Replaces run_ccn_warp_per_shift, run_ccn_warp_per_shift_simple_indexing and

@@ -269,6 +269,7 @@ def make_params(**kw):
 # family -> (entry point stem, kind of matrix-count arguments, caller must zero the output)
 FAMILIES = {
     "overlap_wise": ("xcorr_overlap_wise", "batch", False),
+    "overlap_wise_all_pairs": ("xcorr_overlap_wise_all_pairs", "batch", False),
     "warp_per_overlap": ("xcorr_warp_per_overlap", "pair", None),
     "warp_per_overlap_lds": ("xcorr_warp_per_overlap_lds", "right", None),
     "block_per_overlap": ("xcorr_block_per_overlap", "pair", False),

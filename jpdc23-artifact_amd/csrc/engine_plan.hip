@@ -255,9 +255,17 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     const EngineSpec *best = rq.spec_index > 0 ? &specs[rq.spec_index - 1] : nullptr;
     double best_cost = 0;
     RequestMatch best_match = {};
+    // Several matrices per lane reuse every staged left value, but make a quarter as many work items four times as long:
+    // measured (fp32, 1 x 8 ... 1 x 256 and 2 x 2 ... 32 x 32 matrices of 16x16 ... 256x256) the one-matrix tiles win up to
+    // about 3e9 multiply-adds per launch (by 1.2-1.5x on the smallest), the others beyond; a request for matrices per
+    // thread overrides this.
+    const double pairs = rq.group_m > 0 ? (double)rq.nU : (double)rq.nV * rq.nU;
+    const double area = (double)rq.W * rq.H;
+    const bool one_matrix_per_lane = rq.left_mats <= 1 && rq.right_mats == 0 && pairs * area * area < 3e9;
     for (int i = 0; i < count && rq.spec_index == 0; ++i) {
         const EngineSpec &s = specs[i];
         if (s.A != 1) continue;
+        if (one_matrix_per_lane && s.NV * s.NU > 1) continue;
         if (rq.group_m > 0 && s.NVB() != 1) continue;
         if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
         if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
@@ -277,17 +285,19 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     const bool split_by_default = rq.caller_zeroes ? rq.dist != XCORR_DIST_NONE : rq.may_split;
     if (rc <= 0 && split_by_default) {
         // No chunk size from the caller: the chunk with the lowest relative cost
-        //     (1 + 1300 / (chunk rows x columns)) x (1 + 6.7 x CUs / work items).
+        //     (1 + 1300 / (average rows of a work item x columns)) x (1 + 6.7 x CUs / work items).
         // The first factor is what a work item pays around its sweep (ring start-up, atomic adds of its tile), the second
-        // how badly few items balance over the device. Fitted to measured split-row, multimat-right and multimat-both
-        // launches of 64x64 ... 512x512 fp32 matrices, 1 ... 1024 pairs (it picks 3-5 rows for a single pair up to 96x96,
-        // 8-16 rows around 128x128 ... 512x512, and whole matrices when the pairs alone fill the device).
+        // how badly few items balance over the device; together they put the best number of work items near
+        // sqrt(1.3 x CUs x rows of all tiles x columns). Fitted to measured split-row, multimat-right and multimat-both
+        // launches of 16x16 ... 512x512 fp32 matrices, 1 ... 1024 pairs (3-5 rows for a single pair up to 96x96, 8-16 rows
+        // around 128x128 ... 512x512, whole matrices when the pairs alone fill the device).
         EnginePlan whole;
         if (int e = shape_plan(*best, rq, 0, 1, whole)) return e;
         const double per_tile_column = (double)whole.ntx * whole.nvg * whole.nug;
+        const double rows_of_all_tiles = per_tile_column * count_chunks(*best, rq.H, whole.nty, 1, nullptr);
         auto chunk_cost = [&](int c) {
             const double items = per_tile_column * count_chunks(*best, rq.H, whole.nty, c, nullptr);
-            return (1.0 + 1300.0 / ((double)c * rq.W)) * (1.0 + 6.7 * device_cus() / items);
+            return (1.0 + 1300.0 / (rows_of_all_tiles / items * rq.W)) * (1.0 + 6.7 * device_cus() / items);
         };
         const int candidates[] = {3, 5, 8, 16, 32, 64, rq.H};
         double best_chunk_cost = 0;

@@ -56,23 +56,28 @@ __device__ __forceinline__ void atomic_add_simple(double *p, double v) { unsafeA
 // are added in the order of the definition (row by row, left to right, one accumulator), so a
 // result equals the host loop's bit for bit when that is compiled with the same contraction;
 // eight element pairs are loaded ahead of the eight dependent FMAs so that the loads overlap.
-template <typename T>
+// ALL_PAIRS: every right matrix is correlated with every left matrix, result index = left * batch + right; the strip
+// holds `strip_lefts` result matrices and blockIdx.z walks (group of strip_lefts left matrices, right matrix).
+template <typename T, bool ALL_PAIRS>
 __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__ left, const T *__restrict__ right,
-                                                            T *__restrict__ out, int W, int H, int n_left, int batch) {
+                                                            T *__restrict__ out, int W, int H, int n_left, int batch, int strip_lefts) {
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     const int strip_x = blockIdx.x * blockDim.x + threadIdx.x;
     const int oy = blockIdx.y * blockDim.y + threadIdx.y;
-    const int region = strip_x / Sx;
-    if (region >= n_left || oy >= Sy) return;
-    const int ox = strip_x - region * Sx;
+    const int in_strip = strip_x / Sx;
+    if (in_strip >= strip_lefts || oy >= Sy) return;
+    const int ox = strip_x - in_strip * Sx;
     const int sx = ox - (W - 1), sy = oy - (H - 1);
     const int xl_lo = sx > 0 ? sx : 0, xl_hi = W + sx < W ? W + sx : W;
     const int yl_lo = sy > 0 ? sy : 0, yl_hi = H + sy < H ? H + sy : H;
     const size_t in_area = (size_t)W * H, out_area = (size_t)Sx * Sy;
-    const T *l = left + region * in_area;
-    for (int b = blockIdx.z; b < batch; b += gridDim.z) {
-        const size_t mat = (size_t)b * n_left + region;
-        const T *r = right + mat * in_area;
+    const int steps = ALL_PAIRS ? (n_left / strip_lefts) * batch : batch;
+    for (int z = blockIdx.z; z < steps; z += gridDim.z) {
+        const int b = ALL_PAIRS ? z % batch : z;
+        const int region = ALL_PAIRS ? (z / batch) * strip_lefts + in_strip : in_strip;
+        const size_t mat = ALL_PAIRS ? (size_t)region * batch + b : (size_t)b * n_left + region;
+        const T *l = left + region * in_area;
+        const T *r = right + (ALL_PAIRS ? (size_t)b : mat) * in_area;
         T sum = T(0);
         for (int yl = yl_lo; yl < yl_hi; ++yl) {
             const T *lrow = l + (size_t)yl * W;
@@ -96,23 +101,34 @@ __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__
 
 template <typename T>
 int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
-                     unsigned batch, hipStream_t stream) {
+                     unsigned batch, bool all_pairs, hipStream_t stream) {
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if (n_left == 0 || batch == 0) return fail(XCORR_ERR_INVALID_ARGUMENT, "no matrices");
     if (batch > 0x7fffffffu) return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: batch of %u", batch);
     const unsigned Sx = 2 * cols - 1, Sy = 2 * rows - 1;
     dim3 block(64, 4);
-    unsigned long long strip = (unsigned long long)Sx * n_left;
+    // (all left matrices side by side in the strip: measured faster than one result matrix per strip, which reads the
+    // right matrix of a pair once per left matrix instead of once)
+    const unsigned strip_lefts = n_left;
+    unsigned long long strip = (unsigned long long)Sx * strip_lefts;
     if (strip > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "strip of %u result matrices is too wide", n_left);
-    dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y, batch < 65535 ? batch : 65535);
-    overlap_wise_kernel<T><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch);
+    unsigned long long steps = batch;
+    if (all_pairs) {
+        steps = (unsigned long long)(n_left / strip_lefts) * batch;
+        if ((unsigned long long)n_left * batch > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: %u left, %u right", n_left, batch);
+    }
+    dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y, (unsigned)(steps < 65535 ? steps : 65535));
+    if (all_pairs)
+        overlap_wise_kernel<T, true><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
+    else
+        overlap_wise_kernel<T, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
     XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
-    snprintf(rec.kernel, sizeof(rec.kernel), "overlap_wise/%s", sizeof(T) == 4 ? "f32" : "f64");
+    snprintf(rec.kernel, sizeof(rec.kernel), "overlap_wise/%s%s", sizeof(T) == 4 ? "f32" : "f64", all_pairs ? "_all_pairs" : "");
     rec.block[0] = block.x, rec.block[1] = block.y, rec.block[2] = 1;
-    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = 1;
+    rec.grid[0] = grid.x, rec.grid[1] = grid.y, rec.grid[2] = grid.z;
     rec.y_shifts_per_thread = rec.x_shifts_per_thread = 1;
     rec.left_matrices_per_thread = 1;
     rec.right_matrices_per_thread = batch;

@@ -383,11 +383,19 @@ extern "C" {
 
 int xcorr_overlap_wise_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                            unsigned n_left, unsigned batch, void *stream) {
-    return run_overlap_wise<float>(left, right, out, cols, rows, n_left, batch, as_stream(stream));
+    return run_overlap_wise<float>(left, right, out, cols, rows, n_left, batch, false, as_stream(stream));
 }
 int xcorr_overlap_wise_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                            unsigned n_left, unsigned batch, void *stream) {
-    return run_overlap_wise<double>(left, right, out, cols, rows, n_left, batch, as_stream(stream));
+    return run_overlap_wise<double>(left, right, out, cols, rows, n_left, batch, false, as_stream(stream));
+}
+int xcorr_overlap_wise_all_pairs_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                     unsigned n_left, unsigned n_right, void *stream) {
+    return run_overlap_wise<float>(left, right, out, cols, rows, n_left, n_right, true, as_stream(stream));
+}
+int xcorr_overlap_wise_all_pairs_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
+                                     unsigned n_left, unsigned n_right, void *stream) {
+    return run_overlap_wise<double>(left, right, out, cols, rows, n_left, n_right, true, as_stream(stream));
 }
 
 int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,

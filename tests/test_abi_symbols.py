@@ -19,7 +19,7 @@ def declared_symbols():
 
 def test_header_declares_the_expected_surface():
     names = declared_symbols()
-    for family in ["overlap_wise", "warp_per_overlap", "warp_per_overlap_lds", "block_per_overlap", "shuffle", "split_row", "grouped_overlap", "multimat_right",
+    for family in ["overlap_wise", "overlap_wise_all_pairs", "warp_per_overlap", "warp_per_overlap_lds", "block_per_overlap", "shuffle", "split_row", "grouped_overlap", "multimat_right",
                    "multimat_right_groups", "multimat_right_grouped", "multimat_both", "multimat_both_grouped"]:
         assert f"xcorr_{family}_f32" in names and f"xcorr_{family}_f64" in names
     assert len(names) >= 40

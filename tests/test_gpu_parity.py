@@ -202,6 +202,13 @@ def test_overlap_wise_batches(oracle):
             exp = oracle.n_to_mn(left, right)
             got = xc.run("overlap_wise", left, right, n_left * batch, n_left=n_left, n_right=batch)
             check(got, exp, True, f"overlap_wise {n_left}x{batch}")
+        # every right matrix with every left matrix in one launch (what the reference's host loops over, n_to_m.hpp:198-212)
+        for n_left, n_right, shape in [(1, 4, (7, 9)), (3, 5, (16, 11)), (6, 2, (33, 20)), (3, 4, (10, 70))]:
+            say("overlap_wise all pairs", np.dtype(dtype).name, n_left, n_right, shape)
+            left = ints(rng, (n_left,) + shape, dtype)
+            right = ints(rng, (n_right,) + shape, dtype)
+            got = xc.run("overlap_wise_all_pairs", left, right, n_left * n_right, n_left=n_left, n_right=n_right)
+            check(got, oracle.n_to_m(left, right), True, f"overlap_wise all pairs {n_left}x{n_right}")
 
 
 N_TO_MN_CASES = [
