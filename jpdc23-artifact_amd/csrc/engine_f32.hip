@@ -1,10 +1,10 @@
 // fp32 specialisations of the sliding-window engine (the gfx950-tuned set that
 // replaces the reference's template cross-products, CMakeLists.txt:16-46).
 //
-// Every tile keeps its register budget at or below 128 VGPRs (four wavefronts per SIMD:
-// plain v_fmac_f32 only reaches the vector peak with at least two wavefronts issuing per
-// SIMD, and an even number of resident wavefronts measured best) and its LDS bands at or
-// below ~40 KB per four-wavefront block so four blocks share a CU.
+// Unless its comment says otherwise a tile keeps its register budget at or below 128 VGPRs (four
+// wavefronts per SIMD: plain v_fmac_f32 only reaches the vector peak with at least two wavefronts
+// issuing per SIMD) and its LDS bands at or below ~40 KB per four-wavefront block so four blocks
+// share a CU; the tiles whose comment names 168 registers measured faster with three.
 // Names: a<y shifts>b<x shifts> per lane, r/l = right/left matrices per lane, lr/ll = lanes
 // laid over right/left matrices.
 #include "engine_registry.hpp"

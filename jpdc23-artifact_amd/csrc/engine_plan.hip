@@ -13,7 +13,7 @@ namespace xcorr {
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Relative cost of running a request of the one-output-row families on one of their tiles
-// (their four wavefronts tile 2x2 over the shifts):
+// (their wavefronts tile 2x2 or 1x2 over the shifts):
 //   * work issued for partial overlaps at tile edges: a wavefront skips what cannot overlap its
 //     own tile, but the wavefronts of a block wait for each other after every staged band, so both
 //     the wavefront tile and the block tile count;
