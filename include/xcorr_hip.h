@@ -155,6 +155,11 @@ const char *xcorr_last_error(void);
 int xcorr_last_launch(xcorr_launch_record *out);
 int xcorr_device_info_get(xcorr_device_info *out);
 const char *xcorr_version(void);
+/* Planning without launching (per host thread; no counterpart in the reference): while on, the entry points of the
+ * sliding-window engine (xcorr_shuffle ... xcorr_multimat_both_grouped) validate their arguments, choose kernel and
+ * geometry, fill the launch record and return without launching or reading the pointers. Works without a GPU (256
+ * CUs are assumed then); for tools and tests that ask what a call would run. */
+int xcorr_plan_only(int on);
 
 /* ---- memory / queue shims: the C++ host never includes the HIP headers.
  * They stand in for the reference's cuda_helpers.cuh:26-97 (cuda_malloc,

@@ -399,8 +399,10 @@ int run_engine(const EngineRequest &rq, hipStream_t stream) {
     EnginePlan plan;
     int rc = cached_plan(rq, plan);
     if (rc != XCORR_OK) return rc;
-    rc = rq.elem_bytes == 4 ? launch_typed<float>(rq, plan, stream) : launch_typed<double>(rq, plan, stream);
-    if (rc != XCORR_OK) return rc;
+    if (!plan_only()) {
+        rc = rq.elem_bytes == 4 ? launch_typed<float>(rq, plan, stream) : launch_typed<double>(rq, plan, stream);
+        if (rc != XCORR_OK) return rc;
+    }
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
     snprintf(rec.kernel, sizeof(rec.kernel), "%s/%s", rq.family, plan.spec->name);

@@ -517,8 +517,8 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     const int pitch_l = (int)((cols + 2 * PAD + VK - 1) / VK * VK), pitch_r = (int)((cols + VK - 1) / VK * VK);
     static bool attr_set[64] = {};
     int dev = 0;
-    XCORR_HIP(hipGetDevice(&dev));
-    if (bytes > 64 * 1024 && !(dev >= 0 && dev < 64 && attr_set[dev])) {
+    if (!plan_only()) XCORR_HIP(hipGetDevice(&dev));
+    if (!plan_only() && bytes > 64 * 1024 && !(dev >= 0 && dev < 64 && attr_set[dev])) {
         XCORR_HIP(hipFuncSetAttribute(reinterpret_cast<const void *>(&pair_in_lds_kernel<T, A, B, U, COLS>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                       160 * 1024));
         if (dev >= 0 && dev < 64) attr_set[dev] = true;
@@ -533,8 +533,10 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     auto magic = [](unsigned d) { return (unsigned)((1ull << 32) / d) + 1u; }; // exact for n * d < 2^32, far above any index here
     const PairGeometry geo = {(int)cols,         (int)rows,          pitch_l,       pitch_r, (int)tasks_x, (int)total,
                               magic(pitch_l / VK), magic(pitch_r / VK), magic(tasks_x)};
-    pair_in_lds_kernel<T, A, B, U, COLS><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, geo);
-    XCORR_HIP(hipGetLastError());
+    if (!plan_only()) {
+        pair_in_lds_kernel<T, A, B, U, COLS><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, geo);
+        XCORR_HIP(hipGetLastError());
+    }
     *grid_out = grid;
     *waves_out = waves;
     return XCORR_OK;

@@ -28,6 +28,11 @@ int xcorr_last_launch(xcorr_launch_record *out) {
     return XCORR_OK;
 }
 
+int xcorr_plan_only(int on) {
+    plan_only() = on != 0;
+    return XCORR_OK;
+}
+
 int xcorr_device_info_get(xcorr_device_info *out) {
     if (!out) return fail(XCORR_ERR_INVALID_ARGUMENT, "null info pointer");
     int dev = 0;

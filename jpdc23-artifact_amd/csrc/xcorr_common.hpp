@@ -45,6 +45,11 @@ inline xcorr_launch_record &last_launch() {
     static thread_local xcorr_launch_record rec;
     return rec;
 }
+// Per host thread: plan and record, but do not launch (xcorr_plan_only).
+inline bool &plan_only() {
+    static thread_local bool on = false;
+    return on;
+}
 inline bool &have_last_launch() {
     static thread_local bool have = false;
     return have;

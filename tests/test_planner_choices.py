@@ -1,0 +1,115 @@
+"""CPU-only: what the launcher of the sliding-window engine would run, asked through xcorr_plan_only (the entry
+points validate, plan and fill the launch record without launching; without a GPU the planner assumes 256 CUs).
+Only rules that do not depend on the occupancy the runtime reports for a kernel are pinned here: the tile class a
+family and its tuning integers select, the chunk rule of the one-output-row families, when plain launchers split,
+column chunks, the whole-pair route, and the error paths."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from conftest import load_package
+
+
+class _Dummy:
+    ptr = ctypes.c_void_p(64)  # never read in plan-only mode
+
+
+@pytest.fixture()
+def plan():
+    xc = load_package()
+    lib = xc.lib()
+    assert lib.xcorr_plan_only(1) == 0
+
+    def ask(family, cols, rows, n_left=1, n_right=1, dtype=np.float32, **kw):
+        xc.launch(family, _Dummy, _Dummy, _Dummy, cols, rows, n_left, n_right, dtype, xc.make_params(**kw))
+        return xc.last_launch()
+
+    try:
+        yield ask
+    finally:
+        lib.xcorr_plan_only(0)
+
+
+def test_plain_one_row_launcher_splits_only_when_it_pays(plan):
+    rec = plan("shuffle", 64, 64)
+    assert rec["kernel"] == "shuffle/f32_a1b4" and rec["uses_atomics"] == 1 and 3 <= rec["rows_per_worker"] <= 8
+    rec = plan("shuffle", 64, 64, distribution_type="none")
+    assert rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 64 and rec["distribution_type"] == 1
+    # a large pair: wide tile; "none" keeps it whole whatever the planner would gain
+    rec = plan("shuffle", 1024, 1024, distribution_type="none")
+    assert rec["kernel"] == "shuffle/f32_a1b8" and rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 1024
+    assert plan("shuffle", 512, 512)["kernel"] == "shuffle/f32_a1b8"
+    assert plan("shuffle", 256, 256)["kernel"] == "shuffle/f32_a1b4"
+    assert plan("shuffle", 64, 64, dtype=np.float64)["kernel"] == "shuffle/f64_a1b4"
+
+
+def test_split_row_chunk(plan):
+    # the caller's chunk and distribution are taken as given
+    rec = plan("split_row", 100, 90, rows_per_thread=7, distribution_type="triangle")
+    assert rec["rows_per_worker"] == 7 and rec["distribution_type"] == 3 and rec["uses_atomics"] == 1
+    rec = plan("split_row", 100, 90, rows_per_thread=10)
+    assert rec["rows_per_worker"] == 10 and rec["distribution_type"] == 2  # the reference's default: rectangle
+    # none given: short chunks for one small pair, longer ones as the matrices grow
+    small, medium, large = (plan("split_row", n, n)["rows_per_worker"] for n in (32, 128, 512))
+    assert small <= 5 and 8 <= medium <= 16 and 16 <= large <= 64
+    # rows explicitly whole and few work items: the columns are cut instead
+    rec = plan("split_row", 64, 64, distribution_type="none")
+    assert rec["rows_per_worker"] == 64 and rec["column_chunks"] > 1 and rec["uses_atomics"] == 1
+    rec = plan("split_row", 64, 64, distribution_type="none", column_chunks=1)
+    assert rec["column_chunks"] == 1
+
+
+def test_matrices_per_lane(plan):
+    # small launches: one matrix per lane; a request for matrices per thread overrides; large launches reuse
+    assert plan("multimat_both", 16, 16, 2, 2)["kernel"] == "multimat_both/f32_a1b4"
+    assert plan("multimat_both", 16, 16, 2, 2, right_matrices_per_thread=4)["kernel"] == "multimat_both/f32_a1b4_r4"
+    assert plan("multimat_both", 16, 16, 2, 2, left_matrices_per_thread=2, right_matrices_per_thread=2)["kernel"] == "multimat_both/f32_a1b4_l2r2"
+    rec = plan("multimat_both", 128, 128, 32, 32)
+    assert rec["left_matrices_per_thread"] * rec["right_matrices_per_thread"] > 1
+    assert rec["rows_per_worker"] == 128  # the pairs alone fill the device: whole matrices
+    assert plan("multimat_right", 32, 32, 1, 8)["kernel"] == "multimat_right/f32_a1b4"
+    rec = plan("multimat_right", 256, 256, 1, 32)
+    assert rec["right_matrices_per_thread"] == 4
+
+
+def test_multimat_right_contracts(plan):
+    # plain launcher: may split (then clears the output itself); a distribution or a chunk: the work-distribution contract
+    xc = load_package()
+    assert not xc.needs_zeroed_output("multimat_right", xc.make_params())
+    assert xc.needs_zeroed_output("multimat_right", xc.make_params(distribution_type="triangle"))
+    assert xc.needs_zeroed_output("multimat_right", xc.make_params(rows_per_thread=3))
+    assert not xc.needs_zeroed_output("multimat_right", xc.make_params(distribution_type="none"))
+    rec = plan("multimat_right", 64, 64, 1, 8, distribution_type="triangle")
+    assert rec["uses_atomics"] == 1 and rec["distribution_type"] == 3 and 1 <= rec["rows_per_worker"] < 64
+    rec = plan("multimat_right", 64, 64, 1, 8, distribution_type="none")
+    assert rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 64
+    # the groups entry point plans like the single-left one, over all left matrices
+    one = plan("multimat_right", 64, 64, 1, 4, rows_per_thread=8, distribution_type="rectangle")
+    many = plan("multimat_right_groups", 64, 64, 5, 4, rows_per_thread=8, distribution_type="rectangle")
+    assert many["kernel"] == one["kernel"] and many["grid"][0] == 5 * one["grid"][0]
+
+
+def test_grouped_requests_and_whole_pair_route(plan):
+    assert "pair_in_lds" in plan("grouped_overlap", 64, 64)["kernel"]
+    assert "pair_in_lds" not in plan("grouped_overlap", 64, 64, whole_pair_in_lds=2)["kernel"]
+    assert "pair_in_lds" not in plan("grouped_overlap", 64, 64, shifts_per_thread=8)["kernel"]
+    assert "pair_in_lds" not in plan("grouped_overlap", 300, 300)["kernel"]
+    for asked, got in [(1, 4), (3, 4), (4, 4), (5, 8), (8, 8)]:
+        assert plan("grouped_overlap", 300, 300, shifts_per_thread=asked)["y_shifts_per_thread"] == got
+    rec = plan("multimat_both_grouped", 30, 30, 8, 8, left_matrices_per_thread=4, right_matrices_per_thread=4)
+    assert rec["left_matrices_per_thread"] * rec["lanes_left"] == 4 and rec["right_matrices_per_thread"] * rec["lanes_right"] == 4
+    rec = plan("multimat_right_grouped", 40, 33, 1, 7, shifts_per_thread_right_matrix=2, right_matrices_per_thread=2)
+    assert rec["y_shifts_per_thread"] == 4 and rec["right_matrices_per_thread"] * rec["lanes_right"] == 4
+
+
+def test_errors_in_plan_only_mode(plan):
+    xc = load_package()
+    with pytest.raises(xc.XcorrError, match="Too many shifts per thread: 9"):
+        plan("grouped_overlap", 64, 64, shifts_per_thread=9)
+    with pytest.raises(xc.XcorrError, match="does not exist"):
+        plan("grouped_overlap", 64, 64, specialisation=999)
+    with pytest.raises(xc.XcorrError, match="does not fit the LDS"):
+        plan("grouped_overlap", 300, 300, whole_pair_in_lds=1)
+    with pytest.raises(xc.XcorrError):
+        plan("multimat_right_groups", 16, 16, 3, 0)
