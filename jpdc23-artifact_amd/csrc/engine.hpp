@@ -87,7 +87,29 @@ struct EngineCfg {
     // the same row and column of different bands in one instruction, and an odd stride puts
     // eight such reads on eight different groups of four LDS banks.
     static constexpr int odd_pieces(int n) { return ((n / VK) % 2) ? n : n + VK; }
-    static constexpr int VBAND = odd_pieces((RL + 1) * PV); // one spare row: the last step prefetches past the stage
+    // Left bands, when lanes are laid over left matrices: an LDS pass serves 16 consecutive lanes, i.e. all LX x
+    // positions of up to 16 / LX left bands, and their 128-bit window reads must fall on 16 different groups of four
+    // banks: the pieces lv * (NV * band) + lx * (B / VK) must differ modulo 16. The smallest band size at or above
+    // the rows it has to hold that achieves this is taken (the odd size alone left two-way conflicts on the tiles
+    // with two x lanes: 37 % of the LDS cycles of the fp64 pair tile).
+    static constexpr bool left_reads_collide(int band_elems) {
+        bool seen[16] = {};
+        const int combos = LX * LV < 16 ? LX * LV : 16;
+        for (int c = 0; c < combos; ++c) {
+            const int lx = c % LX, lv = (c / LX) % LV;
+            const int piece = (lv * NV * (band_elems / VK) + lx * (B / VK)) % 16;
+            if (seen[piece]) return true;
+            seen[piece] = true;
+        }
+        return false;
+    }
+    static constexpr int left_band(int n) {
+        if (LV > 1 && LX * (B / VK) <= 16)
+            for (int extra = 0; extra < 16; ++extra)
+                if (!left_reads_collide(n + extra * VK)) return n + extra * VK;
+        return odd_pieces(n);
+    }
+    static constexpr int VBAND = left_band((RL + 1) * PV); // one spare row: the last step prefetches past the stage
     static constexpr int RU = RL + TYB - 1;
     static constexpr int PU = KBX + VK;
     static constexpr int UBAND = odd_pieces((RU + 1) * PU);
