@@ -78,13 +78,15 @@ __device__ __forceinline__ C multiply_conjugate(C a, C b) { // a * conj(b)
     return C{a.x * b.x + a.y * b.y, a.y * b.x - a.x * b.y};
 }
 
-// One thread per element of the reference strip; it walks the `batch` strips of deformed spectra.
+// One thread per element of the reference strip; it walks every gridDim.y-th of the `batch` strips of deformed spectra
+// (the reference's kernel walks all of them, hadamard.cu:34-55: with one small left spectrum and thousands of right ones
+// that is a few hundred threads in a loop of thousands of dependent memory round trips).
 template <typename C>
 __global__ void hadamard_original_kernel(const C *__restrict__ ref, C *__restrict__ deformed, size_t strip, unsigned batch) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= strip) return;
     const C r = ref[i];
-    for (unsigned b = 0; b < batch; ++b) {
+    for (unsigned b = blockIdx.y; b < batch; b += gridDim.y) {
         C *p = deformed + (size_t)b * strip + i;
         *p = multiply_conjugate(r, *p);
     }
@@ -145,7 +147,13 @@ int hadamard_original(const void *ref, void *deformed, unsigned fft_cols, unsign
     if (int rc = check_block(threads)) return rc;
     const size_t strip = (size_t)fft_cols * fft_rows * per_pic;
     if (strip == 0 || batch == 0) return fail(ERR_INVALID_ARGUMENT, "empty hadamard product");
-    hadamard_original_kernel<C><<<grid_for(strip, threads, 1), threads, 0, (hipStream_t)stream>>>((const C *)ref, (C *)deformed, strip, batch);
+    // enough threads to fill the device: the batch is spread over blockIdx.y until about half a million threads exist
+    size_t over_batch = ((size_t)1 << 19) / strip;
+    if (over_batch < 1) over_batch = 1;
+    if (over_batch > batch) over_batch = batch;
+    if (over_batch > 65535) over_batch = 65535;
+    const dim3 grid(grid_for(strip, threads, 1), (unsigned)over_batch);
+    hadamard_original_kernel<C><<<grid, threads, 0, (hipStream_t)stream>>>((const C *)ref, (C *)deformed, strip, batch);
     HIP_CALL(hipGetLastError());
     return OK;
 }
