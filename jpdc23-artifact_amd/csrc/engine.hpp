@@ -65,13 +65,17 @@ struct EngineArgs {
 // DB_ = 1: two sets of LDS bands. While the wavefronts sweep one, the next stage is copied into the
 // other by the memory pipeline itself (loads that write LDS directly, no registers, no waiting
 // wavefront), and one barrier per stage is enough.
+// PG_ = 1 ("paired groups"): the tile serves requests with group_m > 0 only and lays its LV_ lanes over left matrices that
+// each bring their OWN group of right matrices: lane (lv, lu) pairs left matrix v_first + lv with right matrix
+// (v_first + lv) * group_m + ug * LU_ * NU_ + lu * NU_ + n, so the block holds LV_ left bands and LV_ * LU_ * NU_ right bands.
+// With one right matrix per left matrix (independent pairs) no other tile can lay lanes over matrices at all.
 template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_, int LV_, int LU_, int WX_, int WY_,
-          int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0, int SB_ = 8>
+          int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0, int SB_ = 8, int PG_ = 0>
 struct EngineCfg {
     using value_type = T;
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
-    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_, SB = SB_;
+    static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_, SB = SB_, PG = PG_;
     static constexpr int VK = 16 / (int)sizeof(T); // elements per 128-bit LDS access
     static constexpr int TXW = LX * B, TYW = LY * A; // wavefront tile (shifts)
     static constexpr int TXB = TXW * WX, TYB = TYW * WY; // block tile (shifts)
@@ -80,7 +84,9 @@ struct EngineCfg {
     static constexpr int VWIN = B + K - 1;
     static constexpr int VWIN_VECS = (VWIN + VK - 1) / VK;
     static constexpr int KVECS = K / VK;
-    static constexpr int NVB = LV * NV, NUB = LU * NU; // matrices per block
+    static constexpr int NVB = LV * NV;              // left matrices per block
+    static constexpr int NUL = LU * NU;              // right matrices per block that one left matrix meets
+    static constexpr int NUB = PG ? NVB * NUL : NUL; // right bands per block
     // LDS geometry (elements)
     static constexpr int PV = TXB - B + KBX - K + VWIN_VECS * VK;
     // Band sizes are padded to an odd number of 128-bit pieces: lanes laid over matrices read
@@ -120,6 +126,7 @@ struct EngineCfg {
     static constexpr int LDS_BUFFERS = DB ? 2 : 1;
     static constexpr int LDS_BYTES = (LDS_ELEMS * LDS_BUFFERS > RED_ELEMS ? LDS_ELEMS * LDS_BUFFERS : RED_ELEMS) * (int)sizeof(T);
     static_assert(LX * LY * LV * LU == 64, "lane layout must cover one wavefront");
+    static_assert(!PG || NV == 1, "paired groups: one left matrix per lane");
     static_assert(WZ == 1 || (WX == 1 && WY == 1 && (A % WZ == 0 || A < WZ)), "wavefronts that split a reduction share one wavefront tile");
     static_assert((KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
     static_assert(B % VK == 0 && K % VK == 0 && KBX % K == 0 && RL % G == 0, "tile alignment");
@@ -155,9 +162,12 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
 // col_lo <= col < col_hi, and zero otherwise (the caller passes ranges that keep the reads
 // inside the matrices). Every thread moves 128-bit pieces; the loads of up to eight pieces are
 // issued back to back before the first LDS write (C::SB of them), so their latencies overlap.
-template <class C, int NB, int ROWS, int PITCH, int BAND>
-__device__ __forceinline__ void stage_bands(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride, int W,
-                                            int nbands, int row_lo, int row_hi, int row0, int col0, int col_lo, int col_hi, int tid) {
+// (The bands come in groups of NBL: band b is matrix src + (b / NBL) * group_stride + (b % NBL) * mat_stride and exists if
+// b % NBL < nbands and b / NBL < ngroups; a single group when NBL == NB.)
+template <class C, int NB, int NBL, int ROWS, int PITCH, int BAND>
+__device__ __forceinline__ void stage_bands(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride,
+                                            size_t group_stride, int W, int nbands, int ngroups, int row_lo, int row_hi, int row0,
+                                            int col0, int col_lo, int col_hi, int tid) {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     constexpr int VK = C::VK, PP = PITCH / VK, TOTP = NB * ROWS * PP;
@@ -174,8 +184,9 @@ __device__ __forceinline__ void stage_bands(typename C::value_type *lds, const t
             vec v;
 #pragma unroll
             for (int e = 0; e < VK; ++e) v[e] = T(0);
-            if (it0 + j < ITER && band < nbands && row >= row_lo && row < row_hi && col + VK > col_lo && col < col_hi) {
-                const T *q = src + (size_t)band * mat_stride + (size_t)(row0 + row) * W + (ptrdiff_t)(col0 + col);
+            if (it0 + j < ITER && band % NBL < nbands && band / NBL < ngroups && row >= row_lo && row < row_hi && col + VK > col_lo && col < col_hi) {
+                const T *q = src + (size_t)(band / NBL) * group_stride + (size_t)(band % NBL) * mat_stride + (size_t)(row0 + row) * W +
+                             (ptrdiff_t)(col0 + col);
                 if (col >= col_lo && col + VK <= col_hi) {
                     __builtin_memcpy(&v, q, sizeof(vec)); // element-aligned only
                 } else {
@@ -213,10 +224,10 @@ __device__ __forceinline__ void dma_wait() { asm volatile("s_waitcnt vmcnt(0)" :
 // element by element with ordinary stores. The image is addressed linearly in 128-bit pieces
 // (band * BAND/VK + row * PITCH/VK + column piece), which is what makes the 64 pieces of one
 // wavefront-wide copy contiguous in LDS.
-template <class C, int NB, int ROWS, int PITCH, int BAND>
+template <class C, int NB, int NBL, int ROWS, int PITCH, int BAND>
 __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, const typename C::value_type *src, size_t mat_stride,
-                                                  int W, int nbands, int row_lo, int row_hi, int row0, int col0, int col_lo,
-                                                  int col_hi, int tid) {
+                                                  size_t group_stride, int W, int nbands, int ngroups, int row_lo, int row_hi, int row0,
+                                                  int col0, int col_lo, int col_hi, int tid) {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     constexpr int VK = C::VK, PP = PITCH / VK, BANDP = BAND / VK, TOTP = NB * BANDP;
@@ -229,8 +240,9 @@ __device__ __forceinline__ void stage_bands_async(typename C::value_type *lds, c
         const int p = tid + it * C::NT;
         const int band = p / BANDP, q = p % BANDP, row = q / PP, col = (q % PP) * VK;
         if (p < TOTP && row < ROWS) {
-            const bool inside = band < nbands && row >= row_lo && row < row_hi;
-            const T *gp = src + (size_t)band * mat_stride + (ptrdiff_t)(row0 + row) * W + (ptrdiff_t)(col0 + col);
+            const bool inside = band % NBL < nbands && band / NBL < ngroups && row >= row_lo && row < row_hi;
+            const T *gp = src + (size_t)(band / NBL) * group_stride + (size_t)(band % NBL) * mat_stride + (ptrdiff_t)(row0 + row) * W +
+                          (ptrdiff_t)(col0 + col);
             if (inside && col >= col_lo && col + VK <= col_hi) {
                 dma16(gp, lds + (size_t)(wave_piece + it * C::NT) * VK);
             } else {
@@ -414,7 +426,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const int v_first = vg * C::NVB;
     int u_first, u_limit;
     if (g.group_m > 0) {
-        u_first = v_first * g.group_m + ug * C::NUB;
+        // (paired groups: of lane lv = 0; left matrix v_first + lv owns the same slice of its own group, group_m further on)
+        u_first = v_first * g.group_m + ug * C::NUL;
         u_limit = (v_first + 1) * g.group_m;
     } else {
         u_first = ug * C::NUB;
@@ -458,7 +471,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     const int syw = syb + wy * C::TYW;
     const T *Vs_lane = Vs + lv * NV * C::VBAND + wx * C::TXW + lx * B;
     const int lane_ru0 = C::TYB - 1 - (wy * C::TYW + ly * A);
-    const T *Us_lane = Us + lu * NU * C::UBAND + lane_ru0 * C::PU;
+    const T *Us_lane = Us + ((C::PG ? lv * C::NUL : 0) + lu * NU) * C::UBAND + lane_ru0 * C::PU;
 
     T acc[NV][NU][A][B];
 #pragma unroll
@@ -486,21 +499,24 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
         // right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col
         const int yr0 = yl0 - syb - C::TYB + 1;
-        const int nbu = u_limit - u_first < C::NUB ? u_limit - u_first : C::NUB;
+        const int nbu = u_limit - u_first < C::NUL ? u_limit - u_first : C::NUL;
+        // paired groups: one group of right bands per left matrix of the block, group_m matrices apart
+        const int ngu = C::PG ? nbv : 1;
+        const size_t gstride = C::PG ? (size_t)g.group_m * HW : 0;
         const int ur_lo = yr0 < 0 ? -yr0 : 0;
         const int ur_hi = H - yr0 < C::RU + 1 ? H - yr0 : C::RU + 1;
         const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
         T *ubuf = buf + C::NVB * C::VBAND;
         if constexpr (C::DB) {
-            stage_bands_async<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, W, nbv, 0, rows_ok, yl0, xbase,
-                                                                     vc_lo, vc_hi, tid);
-            stage_bands_async<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, W, nbu, ur_lo, ur_hi, yr0, x0,
-                                                                     0, uc_hi, tid);
+            stage_bands_async<C, C::NVB, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, 0, W, nbv, 1, 0, rows_ok, yl0,
+                                                                             xbase, vc_lo, vc_hi, tid);
+            stage_bands_async<C, C::NUB, C::NUL, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, gstride, W, nbu, ngu, ur_lo, ur_hi,
+                                                                             yr0, x0, 0, uc_hi, tid);
         } else {
-            stage_bands<C, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, W, nbv, 0, rows_ok, yl0, xbase, vc_lo,
-                                                               vc_hi, tid);
-            stage_bands<C, C::NUB, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, W, nbu, ur_lo, ur_hi, yr0, x0, 0,
-                                                               uc_hi, tid);
+            stage_bands<C, C::NVB, C::NVB, C::RL + 1, C::PV, C::VBAND>(buf, g.V + (size_t)v_first * HW, HW, 0, W, nbv, 1, 0, rows_ok, yl0, xbase,
+                                                                       vc_lo, vc_hi, tid);
+            stage_bands<C, C::NUB, C::NUL, C::RU + 1, C::PU, C::UBAND>(ubuf, g.U + (size_t)u_first * HW, HW, gstride, W, nbu, ngu, ur_lo, ur_hi, yr0,
+                                                                       x0, 0, uc_hi, tid);
         }
     };
     // this wavefront's part of a staged stage
@@ -617,8 +633,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
                 if (v >= g.nV) continue;
 #pragma unroll
                 for (int n = 0; n < NU; ++n) {
-                    const int u = u_first + lu * NU + n;
-                    if (u >= u_limit) continue;
+                    const int u = u_first + (C::PG ? lv * g.group_m : 0) + lu * NU + n;
+                    if (u >= u_limit + (C::PG ? lv * g.group_m : 0)) continue;
                     const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
                     T *o = g.out + mat_index * out_area + (size_t)oy * Sx;
 #pragma unroll
@@ -641,8 +657,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
         if (v >= g.nV) continue;
 #pragma unroll
         for (int n = 0; n < NU; ++n) {
-            const int u = u_first + lu * NU + n;
-            if (u >= u_limit) continue;
+            const int u = u_first + (C::PG ? lv * g.group_m : 0) + lu * NU + n;
+            if (u >= u_limit + (C::PG ? lv * g.group_m : 0)) continue;
             const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
             T *o = g.out + mat_index * out_area;
 #pragma unroll

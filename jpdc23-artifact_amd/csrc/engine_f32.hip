@@ -49,6 +49,11 @@ using Z_84_v4u8 = EngineCfg<float, 8, 4, 4, 1, 1, 2, 1, 4, 8, 1, 1, 18, 16, 3, 4
 using Z_44_u4 = EngineCfg<float, 4, 4, 4, 1, 1, 4, 4, 1, 4, 1, 1, 20, 16, 4, 4>;
 using Z_44_u8 = EngineCfg<float, 4, 4, 4, 1, 1, 4, 2, 1, 8, 1, 1, 20, 16, 4, 4>;
 
+// paired groups: lanes over 8 left matrices that each bring their own right matrices (n_to_mn with few right matrices per
+// left one, independent pairs); half as many staged rows as the tiles above so that three or four blocks share a CU
+//                                T    A  B  K NV NU  LX LY LV LU  WX WY  RL KBX MINB WZ DB SB PG
+using P_84_p8 = EngineCfg<float, 8, 4, 4, 1, 1, 4, 2, 8, 1, 1, 1, 18, 16, 3, 4, 0, 12, 1>;
+
 static const EngineSpec specs[] = {
     make_spec<R_1x1>("f32_a1b8"),
     make_spec<R_1x4>("f32_a1b8_r4"),
@@ -70,6 +75,7 @@ static const EngineSpec specs[] = {
     make_spec<N_1x1>("f32_a1b4"),
     make_spec<N_1x4>("f32_a1b4_r4"),
     make_spec<N_2x2>("f32_a1b4_l2r2"),
+    make_spec<P_84_p8>("f32_a8b4_pairs8", 0.60, 9.0),
 };
 
 const EngineSpec *engine_specs_f32(int *count) {

@@ -54,8 +54,9 @@ struct RequestMatch {
     bool same_as(const RequestMatch &o) const { return d == o.d; }
 };
 static RequestMatch match_request(const EngineSpec &s, const EngineRequest &rq) {
+    // (the lanes a paired-groups tile lays over left matrices serve different pairs, not several left matrices per thread)
     return RequestMatch{(s.A > 1 ? request_distance(s.A, rq.y_shifts > 1 ? rq.y_shifts : 0) : 0.0) + request_distance(s.NUB(), rq.right_mats) +
-                        request_distance(s.NVB(), rq.left_mats)};
+                        (s.PG ? 0.0 : request_distance(s.NVB(), rq.left_mats))};
 }
 
 // Number of (y tile, chunk) workers when every y tile's rows are cut into chunks of rc rows.
@@ -196,7 +197,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
     for (int i = 0; i < count; ++i) {
         const EngineSpec &s = specs[i];
         if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
-        if (rq.group_m > 0 && s.NVB() != 1) continue;
+        if (rq.group_m > 0 ? (s.NVB() != 1 && !s.PG) : s.PG != 0) continue; // lanes over left matrices: all pairs, or paired groups
         if (rq.spec_index == 0) {
             if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
             if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
@@ -208,7 +209,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         const int longest = rq.W > rq.H ? rq.W : rq.H;
         const bool no_request = rq.spec_index == 0 && rq.y_shifts == 0 && rq.left_mats <= 1 && rq.right_mats == 0 && rq.x_shifts == 0 &&
                                 rq.lanes_x == 0 && rq.lanes_y == 0;
-        if (no_request && s.A > 4 && (longest <= 24 || (longest <= 32 && (rq.group_m > 0 || rq.nV == 1)))) continue;
+        if (no_request && s.A > 4 && (longest <= (s.PG ? 16 : 24) || (longest <= 32 && !s.PG && (rq.group_m > 0 || rq.nV == 1)))) continue;
         const RequestMatch match = match_request(s, rq);
         if (found && best_match.better_than(match)) continue;
         const int G = s.A + 1;
@@ -252,7 +253,10 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     const EngineSpec *specs = rq.elem_bytes == 4 ? engine_specs_f32(&count) : engine_specs_f64(&count);
     if (rq.spec_index > (unsigned)count)
         return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %u does not exist (%d compiled)", rq.family, rq.spec_index, count);
-    if (rq.spec_index > 0 && rq.group_m > 0 && specs[rq.spec_index - 1].NVB() != 1)
+    if (rq.spec_index > 0 && rq.group_m <= 0 && specs[rq.spec_index - 1].PG)
+        return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %s pairs every left matrix with its own group only", rq.family,
+                    specs[rq.spec_index - 1].name);
+    if (rq.spec_index > 0 && rq.group_m > 0 && specs[rq.spec_index - 1].NVB() != 1 && !specs[rq.spec_index - 1].PG)
         return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %s cannot pair one left matrix with a group", rq.family,
                     specs[rq.spec_index - 1].name);
     const bool grouped = rq.spec_index > 0 ? specs[rq.spec_index - 1].A > 1 : rq.y_shifts != 1;
@@ -273,7 +277,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
         const EngineSpec &s = specs[i];
         if (s.A != 1) continue;
         if (one_matrix_per_lane && s.NV * s.NU > 1) continue;
-        if (rq.group_m > 0 && s.NVB() != 1) continue;
+        if (rq.group_m > 0 ? (s.NVB() != 1 && !s.PG) : s.PG != 0) continue; // lanes over left matrices: all pairs, or paired groups
         if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
         if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
         if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;

@@ -19,6 +19,7 @@ struct EngineSpec {
     int LX, LY, LV, LU;
     int WX, WY, RL, KBX;
     int WZ; // wavefronts per workgroup that split one tile's rows and share the LDS bands
+    int PG; // 1: lanes over left matrices that each bring their own group of right matrices (requests with group_m > 0 only)
     int lds_bytes;
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
@@ -34,7 +35,8 @@ struct EngineSpec {
     int TXB() const { return TXW() * WX; }
     int TYB() const { return TYW() * WY; }
     int NVB() const { return LV * NV; }
-    int NUB() const { return LU * NU; }
+    int NUB() const { return LU * NU; } // right matrices per block that one left matrix meets
+    int right_bands() const { return PG ? NVB() * NUB() : NUB(); }
 };
 
 template <class C>
@@ -88,7 +90,7 @@ constexpr EngineSpec make_spec(const char *name, double issue_factor = 1.0, doub
                       C::LU,  C::WX,
                       C::WY,  C::RL,
                       C::KBX, C::WZ,
-                      C::LDS_BYTES,
+                      C::PG,  C::LDS_BYTES,
                       C::NT,  &launch_engine<C>, &resident_blocks_engine<C>, issue_factor, stage_factor};
 }
 

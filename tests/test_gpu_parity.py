@@ -243,6 +243,30 @@ def test_n_to_mn_one_launch(oracle, dtype, kw):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_many_left_matrices_with_few_right_ones_each(oracle, dtype):
+    """n_to_mn with one or two right matrices per left matrix (independent pairs): no tile that lays lanes over the right
+    matrices of ONE left matrix has anything to share, the launcher's pick for thousands of 32x32 fp32 pairs is the tile
+    that lays its lanes over left matrices with their own groups; bit-exact whatever it picks."""
+    xc = load_package()
+    rng = np.random.default_rng(420)
+    picked = set()
+    for n, m, shape in [(2000, 1, (32, 32)), (1000, 2, (32, 32)), (301, 1, (40, 36)), (77, 3, (33, 31)), (1500, 1, (20, 24))]:
+        say("n_to_mn, few right matrices per left", np.dtype(dtype).name, n, m, shape)
+        left = ints(rng, (n,) + shape, dtype)
+        right = ints(rng, (n * m,) + shape, dtype)
+        exp = oracle.n_to_mn(left, right, threads=16)          # file order: right i pairs with left i % n
+        slot = [oracle.interleave_index(i, n * m, n) for i in range(n * m)]
+        right_dev = np.empty_like(right)
+        right_dev[slot] = right
+        got_dev = xc.run("multimat_right_grouped", left, right_dev, n * m, n_left=n, n_right=m)
+        picked.add(xc.last_launch()["kernel"])
+        check(got_dev[slot], exp, True, f"n_to_mn {n}x{m} {shape}")
+    say("kernels:", sorted(picked))
+    if dtype == np.float32:  # (in fp64 that tile measured slower than the single-matrix tiles and is not compiled)
+        assert any("pairs8" in k for k in picked), picked
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("kw", [{}, dict(distribution_type="none"), dict(right_matrices_per_thread=4, distribution_type="rectangle"),
                                 dict(right_matrices_per_thread=2, rows_per_thread=5, distribution_type="triangle"),
                                 dict(rows_per_thread=1, distribution_type="none")], ids=lambda v: str(v).replace(" ", ""))
@@ -329,6 +353,13 @@ def test_every_compiled_specialisation_by_index(oracle):
             left = ints(rng, (n_left,) + shape, dtype)
             right = ints(rng, (n_right,) + shape, dtype)
             cases.append((n_left, n_right, shape, left, right, oracle.n_to_m(left, right, threads=4)))
+        # the tiles that pair every left matrix with its own group of right matrices only serve the n_to_mn layout
+        group_cases = []
+        for n_left, per_left, shape in [(11, 1, (19, 23)), (5, 3, (75, 45)), (9, 2, (33, 40))]:
+            left = ints(rng, (n_left,) + shape, dtype)
+            right = ints(rng, (n_left * per_left,) + shape, dtype)
+            exp = np.concatenate([oracle.one_to_many(left[l:l + 1], right[l * per_left:(l + 1) * per_left]) for l in range(n_left)])
+            group_cases.append((n_left, per_left, shape, left, right, exp))
         index, names = 1, []
         while True:
             try:
@@ -341,8 +372,18 @@ def test_every_compiled_specialisation_by_index(oracle):
                         check(got, exp, True, f"spec {index} {rec['kernel']} rows={rows} {shape}")
                 names.append(rec["kernel"])
             except xc.XcorrError as e:
-                assert "does not exist" in e.message, e
-                break
+                if "own group only" in e.message:
+                    for n_left, per_left, shape, left, right, exp in group_cases:
+                        for rows in (0, 20):
+                            kw = dict(specialisation=index, rows_per_thread=rows)
+                            got = xc.run("multimat_right_grouped", left, right, n_left * per_left, n_left=n_left, n_right=per_left,
+                                         params=xc.make_params(**kw))
+                            rec = xc.last_launch()
+                            check(got, exp, True, f"spec {index} {rec['kernel']} rows={rows} {n_left}x{per_left} {shape}")
+                    names.append(rec["kernel"])
+                else:
+                    assert "does not exist" in e.message, e
+                    break
             index += 1
         say(np.dtype(dtype).name, len(names), "specialisations:", " ".join(n.split("/")[1] for n in names))
         assert len(names) >= 9
