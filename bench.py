@@ -188,8 +188,10 @@ def roofline_of(w, rec, kernel_ms, default_launch):
     achieved = w.flop / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.cfg["dtype"]]
     traffic = MEASURED_TRAFFIC.get((w.name, rec["kernel"])) if default_launch else None
+    # (the fp32 / fp64 MFMA and vector-FMA peaks of MI355X are the same figures)
+    matrix_cores = bool(rec.get("matrix_cores"))
     return {
-        "bound": "valu",
+        "bound": "mfma" if matrix_cores else "valu",
         "achieved": round(achieved, 3),
         "peak": peak,
         "unit": "TFLOP/s",
@@ -323,11 +325,17 @@ def main():
         },
         "roofline": roofline_of(w, rec, kernel_ms, default_launch),
     }
-    result["roofline"]["note"] = (
-        "vector-FMA roofline (MFMA is not used); the kernel issues plain v_fmac_f32, which measures "
-        "0.97 of this peak in a register-only loop on MI355X; the peak assumes 2.4 GHz, the power-managed "
-        "shader clock under this kernel is 2.0-2.1 GHz on random data (2.37 GHz with --data integers)" if dtype == np.float32 else
-        "vector-FMA roofline, v_fma_f64")
+    if result["roofline"]["bound"] == "mfma":
+        result["roofline"]["note"] = (
+            "dense fp32 MFMA roofline (v_mfma_f32_32x32x2_f32: the definition's FMAs only, no padding to a GEMM); the peak assumes "
+            "2.4 GHz, the shader clock under this kernel is 2.35 GHz" if dtype == np.float32 else
+            "dense fp64 MFMA roofline (v_mfma_f64_16x16x4_f64)")
+    else:
+        result["roofline"]["note"] = (
+            "vector-FMA roofline; the kernel issues plain v_fmac_f32, which measures "
+            "0.97 of this peak in a register-only loop on MI355X; the peak assumes 2.4 GHz, the power-managed "
+            "shader clock under this kernel is 2.0-2.1 GHz on random data (2.37 GHz with --data integers)" if dtype == np.float32 else
+            "vector-FMA roofline, v_fma_f64")
 
     if graph_replay:
         result["graph_replay"] = graph_replay

@@ -115,6 +115,9 @@ typedef struct xcorr_params {
     unsigned whole_pair_in_lds;              /* grouped-overlap, one small pair: 0 = the launcher decides, 1 = always run the kernel that
                                                 keeps both matrices in LDS (an error if they do not fit), 2 = never; no counterpart
                                                 in the reference */
+    unsigned matrix_cores;                   /* grouped engine families: 0 = the launcher decides between its register tiles (vector FMA) and
+                                                its matrix-core tiles (v_mfma), 1 = matrix-core tiles only, 2 = never; no counterpart in
+                                                the reference */
 } xcorr_params;
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the
@@ -135,6 +138,8 @@ typedef struct xcorr_launch_record {
     unsigned uses_atomics;     /* 1: partial sums are added with float atomics into a zeroed output */
     unsigned blocks_per_cu;    /* workgroups of this kernel one CU holds at a time (0: not recorded) */
     unsigned column_chunks;    /* chunks the reduction over right columns is cut into (1: not cut) */
+    unsigned matrix_cores;     /* 1: the kernel multiplies on the matrix cores (v_mfma), 0: vector FMAs */
+    float predicted_us;        /* run time the launcher's model expected for the plan it chose (grouped engine families; 0: none) */
 } xcorr_launch_record;
 
 typedef struct xcorr_device_info {

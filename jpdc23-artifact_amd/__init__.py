@@ -52,6 +52,7 @@ class Params(ctypes.Structure):
         ("block_size", ctypes.c_uint),
         ("column_chunks", ctypes.c_uint),
         ("whole_pair_in_lds", ctypes.c_uint),
+        ("matrix_cores", ctypes.c_uint),
     ]
 
 
@@ -76,6 +77,8 @@ class LaunchRecord(ctypes.Structure):
         ("uses_atomics", ctypes.c_uint),
         ("blocks_per_cu", ctypes.c_uint),
         ("column_chunks", ctypes.c_uint),
+        ("matrix_cores", ctypes.c_uint),
+        ("predicted_us", ctypes.c_float),
     ]
 
     def as_dict(self):

@@ -73,6 +73,7 @@ template <typename T, int A_, int B_, int K_, int NV_, int NU_, int LX_, int LY_
           int RL_, int KBX_, int MINB_, int WZ_ = 1, int DB_ = 0, int SB_ = 8, int PG_ = 0>
 struct EngineCfg {
     using value_type = T;
+    static constexpr int MFMA = 0; // (1: the matrix-core sweep of engine_mfma.hpp, a configuration type of its own)
     static constexpr int A = A_, B = B_, K = K_, NV = NV_, NU = NU_;
     static constexpr int LX = LX_, LY = LY_, LV = LV_, LU = LU_;
     static constexpr int WX = WX_, WY = WY_, RL = RL_, KBX = KBX_, MINB = MINB_, WZ = WZ_, DB = DB_, SB = SB_, PG = PG_;
@@ -154,6 +155,103 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
     lo = syb > 0 ? syb : 0;
     int h = syb + C::TYB - 1 + H;
     hi = h < H ? h : H;
+}
+
+// What one workgroup works on: a block tile of shifts, a group of matrices, a chunk of left rows and (when the columns
+// are cut) a chunk of right columns.
+struct WorkItem {
+    int clo, chi;                  // left rows [clo, chi)
+    int syb, sxb;                  // first y / x shift of the block tile
+    int v_first, u_first, u_limit; // first left matrix, first right matrix, end of the right matrices this left group meets
+    int xr_lo, xr_hi, w_hi;        // right columns [xr_lo, xr_hi) to reduce over; w_hi bounds what a partial last stage may sweep
+};
+
+// Decodes blockIdx.x into a work item; false when the block has nothing to do (surplus workers of the rectangle
+// distribution, column chunks beyond a narrow tile's overlap). C supplies the block tile (TXB, TYB), the matrices per
+// block (NVB, NUL, NUB) and the column granule K.
+template <class C, typename T>
+__device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, WorkItem &wi) {
+    const int W = g.W, H = g.H;
+    int item = (int)blockIdx.x;
+    if (item >= g.total_items) return false;
+    const int xch = item % g.x_chunks;
+    item /= g.x_chunks;
+    const int mat = item % (g.nvg * g.nug);
+    item /= (g.nvg * g.nug);
+    const int rc = g.rows_per_chunk;
+    const int worker = item % g.nworkers_y;
+    const int txi = item / g.nworkers_y;
+    const int ug = mat % g.nug, vg = mat / g.nug;
+    // x and y tiles are visited centre-out: the block index order is the dispatch order, and
+    // central tiles have the longest overlaps, so the longest work items start first
+    const int txc = g.ntx / 2, tyc = g.nty / 2;
+    const int tx = (txi & 1) ? txc - (txi + 1) / 2 : txc + txi / 2;
+
+    int tyi, chunk;
+    if (g.dist == 0) {
+        tyi = worker;
+        chunk = 0;
+    } else if (g.dist == 1) {
+        tyi = worker % g.nty;
+        chunk = worker / g.nty;
+    } else {
+        int w = worker;
+        tyi = 0;
+        for (; tyi < g.nty; ++tyi) {
+            int lo, hi;
+            tile_rows<C>((tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2, H, lo, hi);
+            int n = (hi - lo + rc - 1) / rc;
+            if (w < n) break;
+            w -= n;
+        }
+        chunk = w;
+        if (tyi >= g.nty) return false;
+    }
+    const int ty = (tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2;
+    int row_lo, row_hi;
+    tile_rows<C>(ty, H, row_lo, row_hi);
+    wi.clo = row_lo + chunk * rc;
+    wi.chi = wi.clo + rc;
+    if (wi.chi > row_hi) wi.chi = row_hi;
+    if (wi.clo >= wi.chi) return false; // surplus worker of the rectangle distribution
+
+    wi.syb = -(H - 1) + ty * C::TYB;
+    wi.sxb = -(W - 1) + tx * C::TXB;
+
+    // matrices of this block
+    wi.v_first = vg * C::NVB;
+    if (g.group_m > 0) {
+        // (paired groups: of lane lv = 0; left matrix v_first + lv owns the same slice of its own group, group_m further on)
+        wi.u_first = wi.v_first * g.group_m + ug * C::NUL;
+        wi.u_limit = (wi.v_first + 1) * g.group_m;
+    } else {
+        wi.u_first = ug * C::NUB;
+        wi.u_limit = g.nU;
+    }
+
+    // right columns with any overlap for this block tile, from the first K-column chunk that has some on: the first
+    // stage then starts with useful chunks for all wavefronts that split it (aligned to the staging width instead,
+    // the first and the last stage of a tile were both partly empty)
+    int xr_lo = -(wi.sxb + C::TXB - 1);
+    if (xr_lo < 0) xr_lo = 0;
+    xr_lo = (xr_lo / C::K) * C::K;
+    int xr_hi = W - wi.sxb;
+    if (xr_hi > W) xr_hi = W;
+    // this work item's chunk of those columns: [xr_lo, xr_hi) shrinks to it, and w_hi (= W when the
+    // columns are not cut) bounds the columns a partial last stage may sweep
+    wi.w_hi = W;
+    if (g.x_chunks > 1) {
+        const int lo = xr_lo + xch * g.x_chunk_cols;
+        int hi = lo + g.x_chunk_cols;
+        if (hi > xr_hi) hi = xr_hi;
+        if (lo >= hi) return false; // the tile overlaps fewer columns than the widest one
+        xr_lo = lo;
+        xr_hi = hi;
+        wi.w_hi = hi;
+    }
+    wi.xr_lo = xr_lo;
+    wi.xr_hi = xr_hi;
+    return true;
 }
 
 // Fills the LDS image of NB bands (ROWS rows of PITCH elements, BAND elements apart) from NB
@@ -375,85 +473,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
     T *Us = Vs + C::NVB * C::VBAND;
     const int W = g.W, H = g.H;
 
-    // ---- decode the work item (uniform over the threads that share it) ----
-    int item = (int)blockIdx.x;
-    if (item >= g.total_items) return;
-    const int xch = item % g.x_chunks;
-    item /= g.x_chunks;
-    const int mat = item % (g.nvg * g.nug);
-    item /= (g.nvg * g.nug);
-    const int rc = g.rows_per_chunk;
-    const int worker = item % g.nworkers_y;
-    const int txi = item / g.nworkers_y;
-    const int ug = mat % g.nug, vg = mat / g.nug;
-    // x and y tiles are visited centre-out: the block index order is the dispatch order, and
-    // central tiles have the longest overlaps, so the longest work items start first
-    const int txc = g.ntx / 2, tyc = g.nty / 2;
-    const int tx = (txi & 1) ? txc - (txi + 1) / 2 : txc + txi / 2;
-
-    int tyi, chunk;
-    if (g.dist == 0) {
-        tyi = worker;
-        chunk = 0;
-    } else if (g.dist == 1) {
-        tyi = worker % g.nty;
-        chunk = worker / g.nty;
-    } else {
-        int w = worker;
-        tyi = 0;
-        for (; tyi < g.nty; ++tyi) {
-            int lo, hi;
-            tile_rows<C>((tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2, H, lo, hi);
-            int n = (hi - lo + rc - 1) / rc;
-            if (w < n) break;
-            w -= n;
-        }
-        chunk = w;
-        if (tyi >= g.nty) return;
-    }
-    const int ty = (tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2;
-    int row_lo, row_hi;
-    tile_rows<C>(ty, H, row_lo, row_hi);
-    const int clo = row_lo + chunk * rc;
-    int chi = clo + rc;
-    if (chi > row_hi) chi = row_hi;
-    if (clo >= chi) return; // surplus worker of the rectangle distribution
-
-    const int syb = -(H - 1) + ty * C::TYB;
-    const int sxb = -(W - 1) + tx * C::TXB;
-
-    // matrices of this block
-    const int v_first = vg * C::NVB;
-    int u_first, u_limit;
-    if (g.group_m > 0) {
-        // (paired groups: of lane lv = 0; left matrix v_first + lv owns the same slice of its own group, group_m further on)
-        u_first = v_first * g.group_m + ug * C::NUL;
-        u_limit = (v_first + 1) * g.group_m;
-    } else {
-        u_first = ug * C::NUB;
-        u_limit = g.nU;
-    }
-
-    // right columns with any overlap for this block tile, from the first K-column chunk that has some on: the first
-    // stage then starts with useful chunks for all wavefronts that split it (aligned to the staging width instead,
-    // the first and the last stage of a tile were both partly empty)
-    int xr_lo = -(sxb + C::TXB - 1);
-    if (xr_lo < 0) xr_lo = 0;
-    xr_lo = (xr_lo / K) * K;
-    int xr_hi = W - sxb;
-    if (xr_hi > W) xr_hi = W;
-    // this work item's chunk of those columns: [xr_lo, xr_hi) shrinks to it, and w_hi (= W when the
-    // columns are not cut) bounds the columns a partial last stage may sweep
-    int w_hi = W;
-    if (g.x_chunks > 1) {
-        const int lo = xr_lo + xch * g.x_chunk_cols;
-        int hi = lo + g.x_chunk_cols;
-        if (hi > xr_hi) hi = xr_hi;
-        if (lo >= hi) return; // the tile overlaps fewer columns than the widest one
-        xr_lo = lo;
-        xr_hi = hi;
-        w_hi = hi;
-    }
+    // ---- the work item (uniform over the threads that share it) ----
+    WorkItem wi;
+    if (!decode_work_item<C>(g, wi)) return;
+    const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
+    const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
 
     // ---- lane coordinates ----
     const int lane = tid & 63;

@@ -7,6 +7,8 @@
 // share a CU; the tiles whose comment names 168 registers measured faster with three.
 // Names: a<y shifts>b<x shifts> per lane, r/l = right/left matrices per lane, lr/ll = lanes
 // laid over right/left matrices.
+#include <vector>
+
 #include "engine_registry.hpp"
 
 namespace xcorr {
@@ -78,9 +80,17 @@ static const EngineSpec specs[] = {
     make_spec<P_84_p8>("f32_a8b4_pairs8", 0.60, 9.0),
 };
 
+// the register-tile specialisations above followed by the matrix-core ones (engine_mfma_f32.hip): one table, built once
 const EngineSpec *engine_specs_f32(int *count) {
-    *count = (int)(sizeof(specs) / sizeof(specs[0]));
-    return specs;
+    static const std::vector<EngineSpec> all = [] {
+        std::vector<EngineSpec> v(specs, specs + sizeof(specs) / sizeof(specs[0]));
+        int n = 0;
+        const EngineSpec *m = engine_mfma_specs_f32(&n);
+        v.insert(v.end(), m, m + n);
+        return v;
+    }();
+    *count = (int)all.size();
+    return all.data();
 }
 
 } // namespace xcorr

@@ -2,6 +2,8 @@
 // path (its double instantiations are commented out, e.g.
 // naive_shuffle_multirow_both.cu:701-710); these use v_fma_f64 with K = 2 columns per
 // 128-bit LDS access. An 8x8 tile of doubles needs ~190 VGPRs (two wavefronts per SIMD).
+#include <vector>
+
 #include "engine_registry.hpp"
 
 namespace xcorr {
@@ -51,9 +53,17 @@ static const EngineSpec specs[] = {
     make_spec<N_2x2>("f64_a1b4_l2r2_narrow"),
 };
 
+// the register-tile specialisations above followed by the matrix-core ones (engine_mfma_f64.hip): one table, built once
 const EngineSpec *engine_specs_f64(int *count) {
-    *count = (int)(sizeof(specs) / sizeof(specs[0]));
-    return specs;
+    static const std::vector<EngineSpec> all = [] {
+        std::vector<EngineSpec> v(specs, specs + sizeof(specs) / sizeof(specs[0]));
+        int n = 0;
+        const EngineSpec *m = engine_mfma_specs_f64(&n);
+        v.insert(v.end(), m, m + n);
+        return v;
+    }();
+    *count = (int)all.size();
+    return all.data();
 }
 
 } // namespace xcorr

@@ -1,0 +1,353 @@
+// Matrix-core sweep for the grouped families of the sliding-window engine.
+//
+//   out[v,u][sy][sx] = sum over (yl, xr) of V_v[yl][xr+sx] * U_u[yl-sy][xr]
+//
+// For ONE left row yl and a few right columns xr this is a small matrix product whose result does not move as yl and
+// xr advance: D[i][j] += sum_k Ua[i][k] * Vb[k][j] with
+//     i <-> (right matrix u_i, y shift sy_i):   Ua[i][k] = U_{u_i}[yl - sy_i][x_k]      (a window of right rows)
+//     j <-> (left matrix v_j, x shift sx_j):    Vb[k][j] = V_{v_j}[yl][x_k + sx_j]      (a Hankel matrix of one left row)
+// so the whole reduction over (yl, xr) accumulates into the same P x P result tile of v_mfma_f32_32x32x2_f32 (P = 32,
+// two k slots) or v_mfma_f64_16x16x4_f64 (P = 16, four k slots). Nothing is multiplied that the definition does not
+// multiply, except the zero padding at tile edges that the register-tile sweep has as well. Both instructions run at
+// the rate of the vector FMA peak, but one instruction keeps the pipeline busy for 64 / 32 cycles, so the LDS reads
+// and address arithmetic around it are free, and operand reuse happens inside the matrix core instead of in
+// registers: small shift tiles (many matrices per tile) cost nothing extra.
+//
+// Lane l of a wavefront (p = l % P, kk = l / P) supplies row i = p of Ua and column j = p of Vb for k slot kk. The k
+// slots of the EV instructions of a step (4 for the 32 x 32 fp32 tile, 2 for the 16 x 16 fp64 tile) are assigned
+// x_k = x0 + EV * kk + e, e = 0 .. EV-1, so the right operand of a step is ONE aligned LDS read of EV elements per lane
+// and the left operand EV consecutive elements. A step covers 8 right columns with every instruction. The LDS bands, their staging, the work items and the split of a
+// stage's column chunks over the four wavefronts of a block are those of the register-tile sweep (engine.hpp).
+//
+// Result layout of the instructions (lane l, accumulator element r): column j = l % P; row i = 8 * (r / 4) + 4 * (l / 32) + r % 4
+// for the fp32 instruction and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs.
+#pragma once
+
+#include "engine.hpp"
+
+namespace xcorr {
+
+// The instruction of an element type and the layout of its result tile.
+template <typename T>
+struct MfmaOp;
+template <>
+struct MfmaOp<float> {
+    typedef float acc_t __attribute__((ext_vector_type(16)));
+    static constexpr int P = 32, ACC = 16, EV = 4;
+    static constexpr int REG_BITS = 0b11011, LANE_BITS = 0b00100; // which bits of a result row come from the element index / the lane
+    static __device__ __forceinline__ int row(int r, int kk) { return 8 * (r / 4) + 4 * kk + r % 4; } // of element r in lanes l / P = kk
+    static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+};
+template <>
+struct MfmaOp<double> {
+    typedef double acc_t __attribute__((ext_vector_type(4)));
+    static constexpr int P = 16, ACC = 4, EV = 2;
+    static constexpr int REG_BITS = 0b1100, LANE_BITS = 0b0011;
+    static __device__ __forceinline__ int row(int r, int kk) { return 4 * r + kk; }
+    static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
+};
+
+constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 1); }
+
+// JV_ / IU_: left / right matrices laid over the columns / rows of one result tile (P / JV_ x shifts, P / IU_ y shifts).
+// MJX_ x MJV_ result tiles per wavefront along x shifts / further left matrices, NIY_ x NIU_ along y shifts / further
+// right matrices: the wavefront holds MJX_ * MJV_ * NIY_ * NIU_ result tiles and every operand it reads feeds
+// NIY_ * NIU_ (left) or MJX_ * MJV_ (right) instructions.
+// NC_: accumulator sets per result tile. The VK instructions of a step that feed one result tile form a dependent chain;
+// with NC_ > 1 they alternate between NC_ sets that are added up at the end, so a wavefront with few result tiles still
+// has independent instructions in flight (measured on the one-tile fp32 sweep: 0.89 -> 0.96 of the instruction's peak).
+template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int NC_ = 1, int WZ_ = 4, int SB_ = 8>
+struct MfmaCfg {
+    using value_type = T;
+    using Op = MfmaOp<T>;
+    static constexpr int MFMA = 1, PG = 0, DB = 0, SB = SB_;
+    static constexpr int P = Op::P, ACC = Op::ACC, KS = 64 / P;
+    static constexpr int VK = 16 / (int)sizeof(T);
+    static constexpr int EV = Op::EV;   // consecutive elements a lane reads per operand and step = instructions per step and result tile
+    static constexpr int K = KS * EV; // right columns per step (8)
+    static constexpr int JV = JV_, JX = P / JV_, IU = IU_, IY = P / IU_;
+    static constexpr int MJX = MJX_, MJV = MJV_, NIY = NIY_, NIU = NIU_;
+    static constexpr int TJ = MJX * MJV, TI = NIY * NIU; // result tiles of a wavefront
+    static constexpr int TXB = JX * MJX, TYB = IY * NIY, TXW = TXB, TYW = TYB;
+    static constexpr int NVB = JV * MJV, NUL = IU * NIU, NUB = NUL;
+    static constexpr int WX = 1, WY = 1, WZ = WZ_, NWAVES = WZ, NT = 64 * NWAVES;
+    static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_;
+    // what the launch record and the planner call the tile: shifts and matrices per lane, lanes over each
+    static constexpr int A = (1 << popcount_c(Op::REG_BITS & (IY - 1))) * NIY;
+    static constexpr int B = MJX;
+    static constexpr int NV = MJV;
+    static constexpr int NU = (1 << popcount_c(Op::REG_BITS & ~(IY - 1) & (P - 1))) * NIU;
+    static constexpr int LX = JX, LV = JV;
+    static constexpr int LY = 1 << popcount_c(Op::LANE_BITS & (IY - 1));
+    static constexpr int LU = 1 << popcount_c(Op::LANE_BITS & ~(IY - 1));
+    // LDS geometry (elements). Left band: RL rows of every column a shift of the tile can meet in a stage.
+    static constexpr int PV = (TXB + KBX - 1 + VK - 1) / VK * VK;
+    // Lanes p = 0 .. P-1 read element (left matrix p / JX, column p % JX) of one row with one instruction: with the bands
+    // JX (modulo the 256 bytes of the banks) apart they fall on P consecutive banks like the lanes of a single matrix.
+    static constexpr int BANK_ELEMS = 256 / (int)sizeof(T);
+    static constexpr int left_band(int n) {
+        if (JV == 1) return n;
+        int b = n;
+        while (b % BANK_ELEMS != JX % BANK_ELEMS) b += VK;
+        return b;
+    }
+    static constexpr int VBAND = left_band((RL + 1) * PV); // one spare row: the sweep reads one row ahead
+    // Right band: an LDS pass serves the reads of 32 consecutive lanes, and the EV-element pieces they touch must differ
+    // modulo 32 (measured: one collision doubles the pass). Those lanes are rows p = 0 .. P-1 apart and, for the 16-row
+    // tiles, two k slots one piece apart: the row pitch is an odd number of pieces (P = 32) or twice an odd number
+    // (P = 16), and the bands of the IU matrices of a result tile continue the row sequence (band stride = -IY rows
+    // modulo 32 pieces).
+    static constexpr int RU = RL + TYB - 1;
+    static constexpr int right_pitch() {
+        int n = KBX + VK;
+        while (n % VK != 0 || (P == 32 ? (n / EV) % 2 != 1 : (n / EV) % 4 != 2)) n += EV;
+        return n;
+    }
+    static constexpr int PU = right_pitch();
+    static constexpr int right_band(int n) {
+        if (IU == 1) return n;
+        int b = n;
+        while ((b / EV) % 32 != (32 - (IY * (PU / EV)) % 32) % 32) b += VK;
+        return b;
+    }
+    static constexpr int UBAND = right_band((RU + 1) * PU);
+    static constexpr int LDS_ELEMS = NVB * VBAND + NUB * UBAND;
+    // in-block reduction: per pass every wavefront ends up with one quad (four consecutive accumulator elements per lane)
+    static constexpr int NQ = TJ * TI * ACC / 4;
+    static constexpr int QP = WZ < 4 ? WZ : 4; // quads per pass (= wavefronts that add and write in a pass)
+    static constexpr int RED_ELEMS = QP * WZ * 64 * 4;
+    static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
+    static_assert(P % JV == 0 && P % IU == 0, "whole matrices per result tile");
+    static_assert(EV % NC == 0, "the instructions of a step are dealt evenly to the accumulator sets");
+    static_assert(WZ > 1 && (KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
+    static_assert(PV % VK == 0 && VBAND % VK == 0 && UBAND % VK == 0, "128-bit LDS pieces");
+    static_assert(LX * LY * LV * LU == 64, "lane bookkeeping");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+// Wavefront `wave`'s share of one staged stage: column chunks [kc_lo, kc_hi) x left rows [row0, row0 + nrows).
+template <class C>
+__device__ __forceinline__ void mfma_stage(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
+                                           typename C::Op::acc_t (&acc)[C::TJ][C::TI][C::NC], int wave, int kc_lo, int kc_hi, int row0, int nrows) {
+    using T = typename C::value_type;
+    typedef T evec __attribute__((ext_vector_type(C::EV))); // one right-operand read: EV consecutive elements, aligned
+    constexpr int EV = C::EV;
+    auto load = [](const T *vp, const T *up, evec (&a)[C::TI], T (&b)[C::TJ][EV]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < C::TI; ++t)
+            a[t] = *reinterpret_cast<const evec *>(up + (t / C::NIY) * C::IU * C::UBAND - (t % C::NIY) * C::IY * C::PU);
+#pragma unroll
+        for (int s = 0; s < C::TJ; ++s)
+#pragma unroll
+            for (int e = 0; e < EV; ++e) b[s][e] = vp[(s / C::MJX) * C::JV * C::VBAND + (s % C::MJX) * C::JX + e];
+    };
+    auto multiply = [&](const evec (&a)[C::TI], const T (&b)[C::TJ][EV]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < EV; ++e)
+#pragma unroll
+            for (int s = 0; s < C::TJ; ++s)
+#pragma unroll
+                for (int t = 0; t < C::TI; ++t) acc[s][t][e % C::NC] = C::Op::mma(a[t][e], b[s][e], acc[s][t][e % C::NC]);
+    };
+    // A stage whose useful column chunks divide evenly among the WZ wavefronts is dealt chunk by chunk (kc = wave mod WZ).
+    // Otherwise - the tile overlaps only part of the stage's columns, the rule on small matrices - the (chunk, row) steps
+    // are numbered row-fastest and cut into WZ equal runs, so that the wavefronts stay within one step of each other
+    // (dealing whole chunks left three of four idle where a tile overlaps a single chunk of a stage).
+    const int nkc = kc_hi - kc_lo;
+    int kc_a, kc_b, kc_step, j_first, j_last; // chunks kc_a, kc_a + kc_step, ... < kc_b; rows from j_first in the first and up to j_last in the last chunk
+    if (nkc % C::WZ == 0) {
+        kc_a = kc_lo + wave;
+        kc_b = kc_hi;
+        kc_step = C::WZ;
+        j_first = 0;
+        j_last = nrows;
+    } else {
+        const int steps = nkc * nrows;
+        const int first = steps * wave / C::WZ, last = steps * (wave + 1) / C::WZ; // [first, last)
+        if (first >= last) return;
+        kc_a = kc_lo + first / nrows;
+        kc_b = kc_lo + (last - 1) / nrows + 1;
+        kc_step = 1;
+        j_first = first % nrows;
+        j_last = (last - 1) % nrows + 1;
+    }
+    for (int kc = kc_a; kc < kc_b; kc += kc_step) {
+        const int ja = kc == kc_a ? j_first : 0;
+        const int jb = kc + kc_step >= kc_b ? j_last : nrows;
+        const T *vp = Vs_lane + kc * C::K + (row0 + ja) * C::PV;
+        const T *up = Us_lane + kc * C::K + (row0 + ja) * C::PU;
+        // two operand sets: the reads of the next row are issued before the instructions of the current one (the read
+        // past the last row of a sweep lands in the spare row the bands end with and is not used)
+        evec a0[C::TI], a1[C::TI];
+        T b0[C::TJ][EV], b1[C::TJ][EV];
+        load(vp, up, a0, b0);
+        int j = ja;
+#pragma unroll 1
+        for (; j + 2 <= jb; j += 2) {
+            load(vp + C::PV, up + C::PU, a1, b1);
+            multiply(a0, b0);
+            vp += 2 * C::PV;
+            up += 2 * C::PU;
+            load(vp, up, a0, b0);
+            multiply(a1, b1);
+        }
+        if (j < jb) multiply(a0, b0);
+    }
+}
+
+template <class C>
+__global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typename C::value_type> g) {
+    using T = typename C::value_type;
+    using vec = typename vec128<T>::type;
+    using acc_t = typename C::Op::acc_t;
+    constexpr int VK = C::VK, K = C::K, P = C::P;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    const int tid = (int)threadIdx.x;
+    const int group = __builtin_amdgcn_readfirstlane(tid >> 6); // which share of the column chunks
+    T *Vs = reinterpret_cast<T *>(smem_raw);
+    T *Us = Vs + C::NVB * C::VBAND;
+    const int W = g.W, H = g.H;
+
+    WorkItem wi;
+    if (!decode_work_item<C>(g, wi)) return;
+    const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
+    const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
+
+    // ---- lane coordinates inside a result tile ----
+    const int lane = tid & 63;
+    const int p = lane % P, kk = lane / P;
+    const int vj = p / C::JX, sxl = p % C::JX; // column j = p: left matrix, x shift
+    const int ui = p / C::IY, syl = p % C::IY; // row i = p: right matrix, y shift
+    const T *Vs_lane = Vs + vj * C::VBAND + sxl + C::EV * kk;
+    const T *Us_lane = Us + ui * C::UBAND + (C::TYB - 1 - syl) * C::PU + C::EV * kk;
+
+    acc_t acc[C::TJ][C::TI][C::NC];
+#pragma unroll
+    for (int s = 0; s < C::TJ; ++s)
+#pragma unroll
+        for (int t = 0; t < C::TI; ++t)
+#pragma unroll
+            for (int c = 0; c < C::NC; ++c)
+#pragma unroll
+                for (int r = 0; r < C::ACC; ++r) acc[s][t][c][r] = T(0);
+
+    const size_t HW = (size_t)W * H;
+    const int nbv = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
+    const int nbu = u_limit - u_first < C::NUL ? u_limit - u_first : C::NUL;
+
+    // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner). (Fetching the next stage into
+    // registers before the current one is swept, to hide the load latency behind the matrix instructions, measured
+    // 2 % slower on large matrices and no faster on small ones: the other blocks of the CU already cover it.)
+    for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
+        for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
+            __syncthreads(); // everyone is done reading the previous stage
+            {
+                // left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col
+                const int xbase = x0 + sxb;
+                const int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
+                const int vc_lo = xbase < 0 ? -xbase : 0;
+                const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
+                // right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col
+                const int yr0 = yl0 - syb - C::TYB + 1;
+                const int ur_lo = yr0 < 0 ? -yr0 : 0;
+                const int ur_hi = H - yr0 < C::RU ? H - yr0 : C::RU;
+                const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
+                stage_bands<C, C::NVB, C::NVB, C::RL, C::PV, C::VBAND>(Vs, g.V + (size_t)v_first * HW, HW, 0, W, nbv, 1, 0, rows_ok, yl0, xbase, vc_lo,
+                                                                       vc_hi, tid);
+                stage_bands<C, C::NUB, C::NUL, C::RU, C::PU, C::UBAND>(Us, g.U + (size_t)u_first * HW, HW, 0, W, nbu, 1, ur_lo, ur_hi, yr0, x0, 0,
+                                                                       uc_hi, tid);
+            }
+            __syncthreads();
+            // left rows of this stage that can overlap the tile's y shifts: yl in [syb, syb + TYB - 1 + H - 1], yl < chi
+            int first = syb - yl0;
+            int last = syb + C::TYB + H - 2 - yl0;
+            if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
+            if (last > C::RL - 1) last = C::RL - 1;
+            const int row0 = first > 0 ? first : 0;
+            const int nrows = last + 1 - row0;
+            // column chunks of this stage that overlap the tile's x shifts: (x0 + kc*K + K-1) + (sxb + TXB-1) >= 0,
+            // (x0 + kc*K) + sxb <= W-1 and x0 + kc*K < w_hi
+            int kc_lo = 0, kc_hi = C::KBX / K;
+            {
+                int need = -(sxb + C::TXB - 1) - (K - 1) - x0;
+                if (need > 0) kc_lo = (need + K - 1) / K;
+                int lim = W - 1 - sxb - x0;
+                if (w_hi - 1 - x0 < lim) lim = w_hi - 1 - x0;
+                int h = lim < 0 ? 0 : lim / K + 1;
+                if (h < kc_hi) kc_hi = h;
+            }
+            if (nrows > 0 && kc_hi > kc_lo) mfma_stage<C>(Vs_lane, Us_lane, acc, group, kc_lo, kc_hi, row0, nrows);
+        }
+    }
+
+    // ---- add the accumulator sets of every result tile, then the partial tiles of the WZ wavefronts through LDS, and write ----
+#pragma unroll
+    for (int s = 0; s < C::TJ; ++s)
+#pragma unroll
+        for (int t = 0; t < C::TI; ++t)
+#pragma unroll
+            for (int c = 1; c < C::NC; ++c)
+#pragma unroll
+                for (int r = 0; r < C::ACC; ++r) acc[s][t][0][r] += acc[s][t][c][r];
+    // The accumulator elements of a lane are numbered tile * ACC + r and taken in quads of four. In pass q everyone
+    // deposits quads q*QP .. q*QP + QP-1; wavefront w < QP then adds the WZ versions of quad q*QP + w in wavefront order
+    // (deterministic) and writes it: P adjacent x shifts across the lanes.
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
+    const size_t out_area = (size_t)Sx * Sy;
+    T *red = reinterpret_cast<T *>(smem_raw);
+    constexpr int PASSES = (C::NQ + C::QP - 1) / C::QP;
+#pragma unroll
+    for (int q = 0; q < PASSES; ++q) {
+        __syncthreads(); // the bands, or the previous pass, are no longer read
+#pragma unroll
+        for (int o = 0; o < C::QP; ++o) {
+            const int Q = q * C::QP + o;
+            if (Q < C::NQ) {
+                const int tile = Q * 4 / C::ACC, r0 = Q * 4 % C::ACC;
+                T *dst = red + ((size_t)(o * C::WZ + group) * 64 + lane) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; e += VK) {
+                    vec piece;
+#pragma unroll
+                    for (int x = 0; x < VK; ++x) piece[x] = acc[tile / C::TI][tile % C::TI][0][r0 + e + x];
+                    *reinterpret_cast<vec *>(dst + e) = piece;
+                }
+            }
+        }
+        __syncthreads();
+        const int Q = q * C::QP + group;
+        const int tile = Q * 4 / C::ACC, r0 = Q * 4 % C::ACC;
+        const int s = tile / C::TI, t = tile % C::TI;
+        const int v = v_first + (s / C::MJX) * C::JV + vj;
+        const int ox = sxb + (s % C::MJX) * C::JX + sxl + (W - 1);
+        if (group < C::QP && Q < C::NQ && v < g.nV && ox >= 0 && ox < Sx) {
+            T sum[4];
+#pragma unroll
+            for (int src = 0; src < C::WZ; ++src) {
+                const T *from = red + ((size_t)(group * C::WZ + src) * 64 + lane) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; e += VK) {
+                    vec piece = *reinterpret_cast<const vec *>(from + e);
+#pragma unroll
+                    for (int x = 0; x < VK; ++x) sum[e + x] = src == 0 ? piece[x] : sum[e + x] + piece[x];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int i = C::Op::row(r0 + e, kk); // result row: right matrix, y shift
+                const int u = u_first + (t / C::NIY) * C::IU + i / C::IY;
+                const int oy = syb + (t % C::NIY) * C::IY + i % C::IY + (H - 1);
+                if (u < u_limit && oy >= 0 && oy < Sy) {
+                    const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
+                    T *o = g.out + mat_index * out_area + (size_t)oy * Sx + ox;
+                    if (g.atomic)
+                        atomic_add(o, sum[e]);
+                    else
+                        *o = sum[e];
+                }
+            }
+        }
+    }
+}
+
+} // namespace xcorr

@@ -1,0 +1,27 @@
+// fp64 specialisations of the matrix-core sweep (engine_mfma.hpp): v_mfma_f64_16x16x4_f64 result tiles of 16 columns
+// (left matrices x x shifts) by 16 rows (right matrices x y shifts). A wavefront needs at least two result tiles per
+// operand it reads (one tile alone is bound by the LDS reads).
+// Names: m<x shifts>x<y shifts> of the block tile, l / r = left / right matrices per block.
+#include "engine_registry.hpp"
+
+namespace xcorr {
+
+//                               T    JV IU MJX MJV NIY NIU  RL KBX MINB
+using D_32x32 = MfmaCfg<double, 1, 1, 2, 1, 2, 1, 32, 32, 4>;
+using D_32x16 = MfmaCfg<double, 1, 1, 2, 1, 1, 1, 32, 32, 4>;
+using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
+using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 16, 32, 3>;
+
+static const EngineSpec specs[] = {
+    make_spec<D_32x32>("f64_m32x32", 0.75, 1.0),
+    make_spec<D_32x16>("f64_m32x16", 0.80, 1.0),
+    make_spec<D_32x8_r4>("f64_m32x8_r4", 0.78, 1.0),
+    make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.95, 1.0),
+};
+
+const EngineSpec *engine_mfma_specs_f64(int *count) {
+    *count = (int)(sizeof(specs) / sizeof(specs[0]));
+    return specs;
+}
+
+} // namespace xcorr

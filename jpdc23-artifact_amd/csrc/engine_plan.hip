@@ -81,6 +81,7 @@ static long count_chunks(const EngineSpec &s, int H, int nty, int rc, int *max_c
 // chunks (whole shares of the block's wavefronts; ignored where the plan may not add atomically).
 static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int xc, EnginePlan &plan) {
     plan.spec = &s;
+    plan.predicted_us = 0;
     plan.x_chunks = 1;
     plan.x_chunk_cols = rq.W;
     if (xc > 1 && (rq.may_split || rq.caller_zeroes)) {
@@ -152,7 +153,10 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
 // matrices and 1 ... 1024 pairs on MI355X (weighted least squares on the logarithm of the run time);
 // `issue_factor` and `stage_factor` are per tile.
 static double predict_us(const EngineSpec &s, const EngineRequest &rq, const EnginePlan &plan) {
-    const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.LV * s.LU > 1;
+    // (a matrix-core tile lays matrices over the rows and columns of its result tiles: its atomic adds scatter like those of
+    // lanes over matrices; it has no window of A right rows to fill before a chunk's first row)
+    const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.MFMA ? s.NVB() * s.NUB() > 1 : s.LV * s.LU > 1;
+    const int window = s.MFMA ? 0 : s.A - 1;
     const double t_block = 4.41, tau = 1.07, e_full = 0.954, t_stage = 0.209, k_tail = 0.281;
     const double t_clear = f32 ? 1.49 : 0.0, t_atomic = f32 ? 0.0462 : 0.0811;
     const double us_per_atomic = lanes_over_matrices ? (f32 ? 4.5e-6 : 3.0e-6) : (f32 ? 1.6e-6 : 4.4e-6);
@@ -166,8 +170,8 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     const double live = plan.x_chunks > 1 ? std::fmin(plan.x_chunks, std::ceil(cols_tile / plan.x_chunk_cols)) : 1.0;
     const double cols_avg = cols_tile / live, cols_max = plan.x_chunks > 1 ? std::fmin(W, plan.x_chunk_cols) : W;
     const double rows_tile = std::fmin(H, H * (H + TYW) / (plan.nty * TYW));
-    const double rows_avg = (split ? std::fmin(rc, rows_tile) : rows_tile) + s.A - 1;
-    const double rows_max = (split ? rc : H) + s.A - 1;
+    const double rows_avg = (split ? std::fmin(rc, rows_tile) : rows_tile) + window;
+    const double rows_max = (split ? rc : H) + window;
     const double per_element = (double)s.NV * s.NU * s.A * s.B / s.WZ * s.issue_factor;
     const double inst_avg = per_element * rows_avg * cols_avg, inst_max = per_element * rows_max * cols_max;
     const double stages_avg = std::ceil(rows_avg / s.RL) * std::ceil((cols_avg + TXW) / s.KBX) * s.stage_factor;
@@ -176,13 +180,18 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     const int cus = device_cus(), occ = s.resident_blocks();
     double n1 = std::ceil(items / cus);
     if (n1 > occ) n1 = occ;
-    const double fixed = t_block + (split && !lanes_over_matrices ? t_atomic * s.A * s.B : 0.0);
+    const double fixed = t_block + (split && !lanes_over_matrices ? t_atomic * s.NV * s.NU * s.A * s.B : 0.0);
     // n1 blocks on a CU (one wavefront each per SIMD) issue together at e_full * (1 - exp(-n1 / tau)) of the FMA rate
     const double crit = fixed + t_stage * stages_max + n1 * inst_max * cyc / (e_full * (1.0 - std::exp(-n1 / tau)));
     const double per_block = (fixed + t_stage * stages_avg) / n1 + inst_avg * cyc / e_full;
     const double tail = k_tail * crit;
     double t = std::fmax(items * per_block / cus + tail, crit);
-    if (split) t += t_clear + items * 64.0 * s.A * s.B * us_per_atomic;
+    if (split) t += t_clear + items * 64.0 * s.NV * s.NU * s.A * s.B * us_per_atomic;
+    // Sustained vector-FMA load pulls the power-managed shader clock from 2.35 to 2.0-2.1 GHz within the first milliseconds
+    // of a launch (random operands); the matrix cores hold 2.35 GHz on the same data. Measured / predicted run time of the
+    // register tiles is 1.0 below half a millisecond and 1.3 from five milliseconds on, of the matrix-core tiles 1.1
+    // throughout: the register tiles pay the difference, phased in over a decade of run time.
+    if (!s.MFMA && t > 500.0) t *= 1.0 + 0.18 * std::fmin(1.0, std::log10(t / 500.0));
     return t;
 }
 
@@ -199,6 +208,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
         if (rq.group_m > 0 ? (s.NVB() != 1 && !s.PG) : s.PG != 0) continue; // lanes over left matrices: all pairs, or paired groups
         if (rq.spec_index == 0) {
+            if (rq.matrix_cores == 1 ? !s.MFMA : rq.matrix_cores == 2 ? s.MFMA != 0 : false) continue;
             if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
             if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
             if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
@@ -212,7 +222,8 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         if (no_request && s.A > 4 && (longest <= (s.PG ? 16 : 24) || (longest <= 32 && !s.PG && (rq.group_m > 0 || rq.nV == 1)))) continue;
         const RequestMatch match = match_request(s, rq);
         if (found && best_match.better_than(match)) continue;
-        const int G = s.A + 1;
+        const int G = s.MFMA ? 8 : s.A + 1; // granule of the chunk sizes tried
+        const bool matrices_in_tile = s.MFMA ? s.NVB() * s.NUB() > 1 : s.LV * s.LU > 1;
         for (int k : ladder) {
             int rc = k * G;
             if (rq.rows_per_worker > 0 || rq.caller_zeroes) {
@@ -220,7 +231,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
                 rc = (int)rq.rows_per_worker;
             } else if (k != 0 && (!rq.may_split || rc >= rq.H)) {
                 break;
-            } else if (k != 0 && s.LV * s.LU > 1 && (rc < 36 || rq.H < 72)) {
+            } else if (k != 0 && matrices_in_tile && (rc < 36 || rq.H < 72)) {
                 continue; // measured: short chunks of tiles whose lanes lie over matrices lose to their scattered atomic adds
             }
             EnginePlan cand;
@@ -231,6 +242,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
                 best = t;
                 best_match = match;
                 plan = cand;
+                plan.predicted_us = t;
             }
         }
     }
@@ -240,7 +252,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
     // A split plan that still leaves CUs without a block (a single pair of 32x32 ... 64x64 matrices) also cuts the
     // reduction over right columns in two: measured 12-20 % faster there, slower as soon as every CU has a block
     // (the model above was not fitted for column chunks and is not asked).
-    if (rq.column_chunks == 0 && plan.zero_fill && plan.spec->LV * plan.spec->LU == 1 && plan.total_items < device_cus() && rq.W >= 32) {
+    if (rq.column_chunks == 0 && plan.zero_fill && plan.spec->LV * plan.spec->LU == 1 && !plan.spec->MFMA && plan.total_items < device_cus() && rq.W >= 32) {
         EnginePlan cut;
         if (int e = shape_plan(*plan.spec, rq, plan.rows_per_chunk, 2, cut)) return e;
         plan = cut;
@@ -251,6 +263,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
 int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     int count = 0;
     const EngineSpec *specs = rq.elem_bytes == 4 ? engine_specs_f32(&count) : engine_specs_f64(&count);
+    if (rq.matrix_cores > 2) return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: matrix_cores must be 0, 1 or 2, not %u", rq.family, rq.matrix_cores);
     if (rq.spec_index > (unsigned)count)
         return fail(XCORR_ERR_INVALID_ARGUMENT, "%s: specialisation %u does not exist (%d compiled)", rq.family, rq.spec_index, count);
     if (rq.spec_index > 0 && rq.group_m <= 0 && specs[rq.spec_index - 1].PG)
@@ -379,7 +392,7 @@ static bool same_shape(const EngineRequest &a, const EngineRequest &b) {
     return strcmp(a.family, b.family) == 0 && a.elem_bytes == b.elem_bytes && a.W == b.W && a.H == b.H && a.nV == b.nV && a.nU == b.nU &&
            a.group_m == b.group_m && a.y_shifts == b.y_shifts && a.x_shifts == b.x_shifts && a.left_mats == b.left_mats &&
            a.right_mats == b.right_mats && a.lanes_x == b.lanes_x && a.lanes_y == b.lanes_y && a.waves == b.waves &&
-           a.spec_index == b.spec_index && a.rows_per_worker == b.rows_per_worker && a.column_chunks == b.column_chunks &&
+           a.spec_index == b.spec_index && a.rows_per_worker == b.rows_per_worker && a.column_chunks == b.column_chunks && a.matrix_cores == b.matrix_cores &&
            a.dist == b.dist && a.caller_zeroes == b.caller_zeroes && a.may_split == b.may_split;
 }
 
@@ -437,6 +450,8 @@ int run_engine(const EngineRequest &rq, hipStream_t stream) {
     rec.uses_atomics = plan.atomic;
     rec.blocks_per_cu = plan.spec->resident_blocks();
     rec.column_chunks = plan.x_chunks;
+    rec.matrix_cores = plan.spec->MFMA;
+    rec.predicted_us = (float)plan.predicted_us;
     have_last_launch() = true;
     return XCORR_OK;
 }

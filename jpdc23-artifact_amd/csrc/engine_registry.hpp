@@ -8,6 +8,7 @@
 #pragma once
 
 #include "engine.hpp"
+#include "engine_mfma.hpp"
 #include "xcorr_common.hpp"
 
 namespace xcorr {
@@ -20,6 +21,7 @@ struct EngineSpec {
     int WX, WY, RL, KBX;
     int WZ; // wavefronts per workgroup that split one tile's rows and share the LDS bands
     int PG; // 1: lanes over left matrices that each bring their own group of right matrices (requests with group_m > 0 only)
+    int MFMA; // 1: matrix-core sweep (engine_mfma.hpp); A, B, NV, NU, L* then describe what a lane holds of the result tiles
     int lds_bytes;
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
@@ -39,6 +41,15 @@ struct EngineSpec {
     int right_bands() const { return PG ? NVB() * NUB() : NUB(); }
 };
 
+// the kernel a configuration type stands for
+template <class C>
+constexpr auto kernel_of() {
+    if constexpr (C::MFMA != 0)
+        return &mfma_kernel<C>;
+    else
+        return &engine_kernel<C>;
+}
+
 template <class C>
 hipError_t allow_large_lds() {
     if (C::LDS_BYTES <= 64 * 1024) return hipSuccess;
@@ -48,7 +59,7 @@ hipError_t allow_large_lds() {
     if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
     const bool tracked = dev >= 0 && dev < 64;
     if (!tracked || !attr_set[dev]) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&engine_kernel<C>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel_of<C>()),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return e;
         if (tracked) attr_set[dev] = true;
@@ -60,7 +71,7 @@ template <class C>
 hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
     using T = typename C::value_type;
     if (hipError_t e = allow_large_lds<C>(); e != hipSuccess) return e;
-    engine_kernel<C><<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
+    kernel_of<C>()<<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
     return hipGetLastError();
 }
 
@@ -71,7 +82,7 @@ int resident_blocks_engine() {
     if (blocks[dev] == 0) {
         int n = 0;
         if (allow_large_lds<C>() != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(&engine_kernel<C>), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
             (void)hipGetLastError();
             n = 1;
         }
@@ -90,13 +101,16 @@ constexpr EngineSpec make_spec(const char *name, double issue_factor = 1.0, doub
                       C::LU,  C::WX,
                       C::WY,  C::RL,
                       C::KBX, C::WZ,
-                      C::PG,  C::LDS_BYTES,
+                      C::PG,  C::MFMA, C::LDS_BYTES,
                       C::NT,  &launch_engine<C>, &resident_blocks_engine<C>, issue_factor, stage_factor};
 }
 
 // defined in engine_f32.hip / engine_f64.hip
 const EngineSpec *engine_specs_f32(int *count);
 const EngineSpec *engine_specs_f64(int *count);
+// defined in engine_mfma_f32.hip / engine_mfma_f64.hip: the matrix-core specialisations, appended to the tables above
+const EngineSpec *engine_mfma_specs_f32(int *count);
+const EngineSpec *engine_mfma_specs_f64(int *count);
 
 // What a family asks of the engine.
 struct EngineRequest {
@@ -111,6 +125,7 @@ struct EngineRequest {
     unsigned spec_index;      // 1-based: use exactly this entry of the specialisation table
     unsigned rows_per_worker; // 0 = planner decides
     unsigned column_chunks;   // 0 = planner decides (grouped families only)
+    unsigned matrix_cores;    // 0 = planner decides, 1 = matrix-core tiles only, 2 = register tiles only
     unsigned dist;            // XCORR_DIST_*
     bool caller_zeroes;       // true: split-row contract, output arrives zeroed, always accumulate atomically
     bool may_split;           // planner may split the reduction and clear the output itself
@@ -123,6 +138,7 @@ struct EnginePlan {
     int x_chunks, x_chunk_cols; // chunks of right columns per tile (1: not cut) and their width
     bool zero_fill;
     unsigned grid;
+    double predicted_us; // of the run-time model (grouped families; 0 where no model was asked)
 };
 
 int plan_engine(const EngineRequest &rq, EnginePlan &plan);

@@ -222,6 +222,7 @@ EngineRequest base_request(const char *family, int elem_bytes, const void *left,
     rq.lanes_y = p.lanes_y;
     rq.spec_index = p.specialisation;
     rq.column_chunks = p.column_chunks;
+    rq.matrix_cores = p.matrix_cores;
     rq.waves = waves_from_warps(p.warps_per_thread_block);
     rq.dist = p.distribution_type;
     return rq;

@@ -127,7 +127,7 @@ def test_tuning_integers_select_tiles(tmp_path, oracle):
         seen[label] = dict(zip(header.split(","), row.split(",")))["shifts_per_thread"]
         np.testing.assert_array_equal(read_matrices(tmp_path / f"{label}_o.csv")[0], exp[0], err_msg=label)
     assert seen["four"] == "4" and seen["three"] == "4" and seen["eight"] == "8" and seen["five"] == "8", seen
-    assert seen["none"] in ("4", "8")
+    assert seen["none"] in ("4", "8", "16")  # 16: the matrix-core tile, a lane holds 16 y shifts of its 32 x 32 result tile
     # n_to_m: matrices per thread pick the lanes-over-matrices tiles
     left = rng.integers(-3, 4, (8, 30, 30)).astype(np.float32)
     right = rng.integers(-3, 4, (8, 30, 30)).astype(np.float32)
