@@ -278,7 +278,7 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     // 32: 3.9 / 7.4, 64: 6.0 / 10.4, 80: 11.2 / 12.6, 96: 14.1 / 16.1, 112: 19.0 / 21.0, 128: 28.6 / 21.6; fp64 32: 4.4 / 8.0,
     // 64: 8.6 / 13.1, 96: 19.2 / 23.3. Beyond the sizes below the engine's register tiles win.
     const bool tile_asked = p.specialisation || p.x_shifts_per_thread || p.lanes_x || p.lanes_y || p.rows_per_thread || p.column_chunks ||
-                            p.shifts_per_thread || p.distribution_type != XCORR_DIST_DEFAULT;
+                            p.shifts_per_thread || p.matrix_cores || p.distribution_type != XCORR_DIST_DEFAULT;
     const size_t elems = (size_t)cols * rows;
     const bool small = pair_fits_lds<T>(cols, rows) && cols <= 128 && elems <= (sizeof(T) == 4 ? 112u * 112u : 96u * 96u);
     if (p.whole_pair_in_lds == 1 || (p.whole_pair_in_lds == 0 && !tile_asked && small))

@@ -1,0 +1,117 @@
+"""GPU parity of the matrix-core tiles (xcorr_params.matrix_cores = 1 keeps the launcher to them): every mode of the
+grouped families on shapes that do not divide the 32 x 32 / 16 x 16 result tiles, the 8-column steps or the staged bands,
+whole and with the reduction cut into atomically added chunks of rows and columns, against the CPU oracle.
+Integer-valued inputs must match bit for bit, real-valued ones to 1e-5 (fp32) / 1e-12 (fp64) relative Frobenius error."""
+import numpy as np
+import pytest
+
+from conftest import load_package
+
+pytestmark = pytest.mark.gpu
+
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+SHAPES = [(1, 1), (1, 9), (7, 1), (5, 3), (16, 16), (31, 33), (33, 17), (64, 64), (70, 130), (150, 41)]
+CHUNKINGS = [{}, dict(rows_per_thread=8), dict(rows_per_thread=24, distribution_type="rectangle"), dict(rows_per_thread=40, column_chunks=2),
+             dict(distribution_type="none")]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def ints(rng, shape, dtype, amp=4):
+    return rng.integers(-amp, amp + 1, size=shape).astype(dtype)
+
+
+def rel_frob(a, b):
+    a, b = a.astype(np.float64).ravel(), b.astype(np.float64).ravel()
+    den = np.linalg.norm(b)
+    return np.linalg.norm(a - b) / (den if den > 0 else 1.0)
+
+
+def launch_and_check(xc, family, left, right, n_results, n_left, n_right, exp, exact, kw, seen):
+    got = xc.run(family, left, right, n_results, n_left=n_left, n_right=n_right, params=xc.make_params(matrix_cores=1, **kw))
+    rec = xc.last_launch()
+    what = f"{family} {left.shape} x {right.shape} {kw} {rec['kernel']} rows={rec['rows_per_worker']} atomics={rec['uses_atomics']}"
+    assert rec["matrix_cores"] == 1, what
+    seen.add(rec["kernel"].split("/")[1])
+    assert np.isfinite(got).all(), what
+    if exact:
+        bad = np.argwhere(got != exp)
+        assert bad.size == 0, f"{what}: {len(bad)} elements differ, first {bad[:3].tolist()}"
+    else:
+        err = rel_frob(got, exp)
+        assert err <= TOL[got.dtype], f"{what}: rel frobenius {err:.3e}"
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_one_pair(oracle, dtype):
+    xc = load_package()
+    rng = np.random.default_rng(900)
+    seen = set()
+    for shape in SHAPES + [(200, 260)]:
+        left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
+        exp = oracle.one_to_one(left, right, threads=4)
+        for kw in CHUNKINGS:
+            say("one pair", np.dtype(dtype).name, shape, kw)
+            launch_and_check(xc, "grouped_overlap", left, right, 1, 1, 1, exp, True, kw, seen)
+    left, right = rng.standard_normal((130, 150)).astype(dtype), rng.standard_normal((130, 150)).astype(dtype)
+    launch_and_check(xc, "grouped_overlap", left, right, 1, 1, 1, oracle.one_to_one(left, right, threads=4), False, {}, seen)
+    say(sorted(seen))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_one_to_many_and_groups(oracle, dtype):
+    xc = load_package()
+    rng = np.random.default_rng(901)
+    seen = set()
+    for shape in [(1, 1), (5, 3), (16, 16), (33, 17), (40, 70), (64, 64)]:
+        for n_right in (1, 3, 4, 9, 17):
+            left, right = ints(rng, (1,) + shape, dtype), ints(rng, (n_right,) + shape, dtype)
+            exp = oracle.one_to_many(left, right)
+            for kw in CHUNKINGS[:3] + [dict(right_matrices_per_thread=4)]:
+                say("one_to_many", np.dtype(dtype).name, shape, n_right, kw)
+                launch_and_check(xc, "multimat_right_grouped", left, right, n_right, 1, n_right, exp, True, kw, seen)
+        # every left matrix with its own group of right matrices, one launch
+        for n_left, per_left in [(2, 1), (3, 5), (7, 4), (4, 9)]:
+            left, right = ints(rng, (n_left,) + shape, dtype), ints(rng, (n_left * per_left,) + shape, dtype)
+            exp = np.concatenate([oracle.one_to_many(left[l:l + 1], right[l * per_left:(l + 1) * per_left]) for l in range(n_left)])
+            for kw in CHUNKINGS[:2]:
+                say("n_to_mn", np.dtype(dtype).name, shape, n_left, per_left, kw)
+                launch_and_check(xc, "multimat_right_grouped", left, right, n_left * per_left, n_left, per_left, exp, True, kw, seen)
+    left, right = rng.random((1, 90, 75)).astype(dtype), rng.random((6, 90, 75)).astype(dtype)
+    launch_and_check(xc, "multimat_right_grouped", left, right, 6, 1, 6, oracle.one_to_many(left, right, threads=4), False, {}, seen)
+    say(sorted(seen))
+    assert any("_r" in k for k in seen), seen  # tiles with right matrices over the rows of a result tile were used
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_all_pairs(oracle, dtype):
+    xc = load_package()
+    rng = np.random.default_rng(902)
+    seen = set()
+    for shape in [(1, 1), (3, 5), (16, 16), (19, 23), (33, 40), (64, 64)]:
+        for n_left, n_right in [(1, 1), (2, 3), (4, 4), (5, 9), (9, 5), (13, 2)]:
+            left, right = ints(rng, (n_left,) + shape, dtype), ints(rng, (n_right,) + shape, dtype)
+            exp = oracle.n_to_m(left, right, threads=4)
+            for kw in CHUNKINGS[:3] + [dict(left_matrices_per_thread=4, right_matrices_per_thread=4)]:
+                say("n_to_m", np.dtype(dtype).name, shape, n_left, n_right, kw)
+                launch_and_check(xc, "multimat_both_grouped", left, right, n_left * n_right, n_left, n_right, exp, True, kw, seen)
+    left, right = rng.standard_normal((5, 50, 60)).astype(dtype), rng.standard_normal((7, 50, 60)).astype(dtype)
+    launch_and_check(xc, "multimat_both_grouped", left, right, 35, 5, 7, oracle.n_to_m(left, right, threads=4), False, {}, seen)
+    say(sorted(seen))
+    assert any("_l" in k for k in seen), seen  # tiles with left matrices over the columns of a result tile were used
+
+
+def test_never_and_only(oracle):
+    """matrix_cores = 2 keeps the register tiles; both settings give the same integers."""
+    xc = load_package()
+    rng = np.random.default_rng(903)
+    left, right = ints(rng, (300, 280), np.float32), ints(rng, (300, 280), np.float32)
+    exp = oracle.one_to_one(left, right, threads=4)
+    for setting, flag in [(1, 1), (2, 0)]:
+        got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(matrix_cores=setting))
+        assert xc.last_launch()["matrix_cores"] == flag
+        assert np.array_equal(got, exp)
+    with pytest.raises(xc.XcorrError, match="matrix_cores must be 0, 1 or 2"):
+        xc.run("grouped_overlap", left, right, 1, params=xc.make_params(matrix_cores=7))

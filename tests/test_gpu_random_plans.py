@@ -33,6 +33,8 @@ def draw_params(rng, family, rows):
         kw["warps_per_thread_block"] = int(rng.choice([1, 4, 8, 32]))
     if "grouped" in family:
         if rng.random() < 0.5:
+            kw["matrix_cores"] = int(rng.choice([1, 2]))
+        if rng.random() < 0.5:
             key = "shifts_per_thread" if family == "grouped_overlap" else "shifts_per_thread_right_matrix"
             kw[key] = int(rng.integers(1, 9 if family == "grouped_overlap" else 5))
         if rng.random() < 0.3:

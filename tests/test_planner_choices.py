@@ -103,6 +103,30 @@ def test_grouped_requests_and_whole_pair_route(plan):
     assert rec["y_shifts_per_thread"] == 4 and rec["right_matrices_per_thread"] * rec["lanes_right"] == 4
 
 
+def test_matrix_core_tiles(plan):
+    # a large pair runs on the matrix cores by default; matrix_cores = 2 keeps the register tiles, 1 excludes them
+    rec = plan("grouped_overlap", 1024, 1024)
+    assert rec["matrix_cores"] == 1 and rec["kernel"].startswith("grouped_overlap/f32_m") and rec["predicted_us"] > 0
+    assert rec["lanes_x"] * rec["lanes_y"] * rec["lanes_left"] * rec["lanes_right"] == 64
+    rec = plan("grouped_overlap", 1024, 1024, matrix_cores=2)
+    assert rec["matrix_cores"] == 0 and rec["kernel"] == "grouped_overlap/f32_a8b4"
+    rec = plan("grouped_overlap", 512, 512, dtype=np.float64, matrix_cores=1)
+    assert rec["matrix_cores"] == 1 and "f64_m32x" in rec["kernel"]
+    # one left matrix with its own right matrices: only tiles with a single left matrix; all pairs: any
+    rec = plan("multimat_right_grouped", 128, 128, 8, 16, matrix_cores=1)
+    assert rec["matrix_cores"] == 1 and rec["left_matrices_per_thread"] * rec["lanes_left"] == 1
+    rec = plan("multimat_both_grouped", 64, 64, 16, 32, matrix_cores=1)
+    assert rec["matrix_cores"] == 1
+    # the reference's tuning integers still restrict the choice: eight y shifts per thread exist among the register tiles only
+    rec = plan("grouped_overlap", 300, 300, shifts_per_thread=8)
+    assert rec["matrix_cores"] == 0 and rec["y_shifts_per_thread"] == 8
+    xc = load_package()
+    with pytest.raises(xc.XcorrError, match="matrix_cores must be 0, 1 or 2"):
+        plan("grouped_overlap", 300, 300, matrix_cores=3)
+    # the one-output-row families have no matrix-core tiles
+    assert plan("split_row", 256, 256)["matrix_cores"] == 0
+
+
 def test_errors_in_plan_only_mode(plan):
     xc = load_package()
     with pytest.raises(xc.XcorrError, match="Too many shifts per thread: 9"):
