@@ -125,6 +125,87 @@ struct MfmaCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
+// Staging of NB bands (ROWS rows x COLS columns each; row pitch PITCH and band stride BAND in LDS; matrices `mat_stride`
+// apart in global memory) with everything that does not change from stage to stage worked out once per block: thread
+// `tid` moves the 128-bit pieces p = tid + i * NT, piece p being (band, row, column piece) = (p / (PP * ROWS),
+// (p / PP) % ROWS, p % PP), and keeps per piece its byte offset from the stage's origin in global memory, its LDS offset
+// and its coordinates. A stage that lies wholly inside the matrices (the rule away from the matrix edges) is then one
+// load with a scalar base and one LDS store per piece, no address arithmetic; the other stages zero what lies outside
+// [row_lo, row_hi) x [col_lo, col_hi) or belongs to a band that does not exist and assemble pieces that straddle a column
+// bound element by element. (Every instruction a wavefront issues next to the matrix instructions of the other
+// wavefronts of its SIMD costs the matrix pipeline about two cycles; the generic staging of the register-tile sweep
+// issued as many vector and scalar instructions per stage as the sweep issues matrix instructions.)
+template <class C, int NB, int ROWS, int COLS, int PITCH, int BAND>
+struct BandStager {
+    using T = typename C::value_type;
+    using vec = typename vec128<T>::type;
+    static constexpr int VK = C::VK, PP = COLS / VK, TOTP = NB * ROWS * PP;
+    static constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
+    static constexpr int BATCH = ITER < C::SB ? ITER : C::SB;
+    static constexpr unsigned NONE = ~0u;
+    static_assert(COLS % VK == 0 && PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
+    static_assert(ROWS < 4096 && COLS <= 4096 && NB < 255, "packed piece coordinates");
+    unsigned gbyte[ITER]; // byte offset of the piece from the stage origin (the element at band 0, row 0, column 0)
+    unsigned where[ITER]; // band << 24 | row << 12 | column; NONE: this thread has no piece in this round
+    int lds_at[ITER];     // element offset in the LDS image
+    __device__ __forceinline__ void init(int tid, int W, size_t mat_stride) {
+#pragma unroll
+        for (int i = 0; i < ITER; ++i) {
+            const int p = tid + i * C::NT;
+            const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
+            const bool have = p < TOTP;
+            gbyte[i] = have ? (unsigned)(((size_t)band * mat_stride + (size_t)row * W + col) * sizeof(T)) : 0u;
+            where[i] = have ? ((unsigned)band << 24 | (unsigned)row << 12 | (unsigned)col) : NONE;
+            lds_at[i] = have ? band * BAND + row * PITCH + col : 0;
+        }
+    }
+    // `origin`: address of (band 0, row 0, column 0) of the stage; it may lie outside the matrix where the bounds exclude
+    // the elements there (it is only offset, never read through, for those)
+    __device__ __forceinline__ void stage(T *lds, const T *origin, int nbands, int row_lo, int row_hi, int col_lo, int col_hi) const {
+        const char *base = reinterpret_cast<const char *>(origin);
+        const bool interior = nbands >= NB && row_lo <= 0 && row_hi >= ROWS && col_lo <= 0 && col_hi >= COLS;
+#pragma unroll
+        for (int i0 = 0; i0 < ITER; i0 += BATCH) {
+            vec val[BATCH];
+            if (interior) {
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j) {
+                    const int i = i0 + j;
+                    if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) __builtin_memcpy(&val[j], base + gbyte[i], sizeof(vec)); // element-aligned only
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < BATCH; ++j) {
+                    const int i = i0 + j;
+                    vec v;
+#pragma unroll
+                    for (int e = 0; e < VK; ++e) v[e] = T(0);
+                    if (i < ITER) {
+                        const unsigned w = where[i];
+                        const int col = (int)(w & 0xFFFu), row = (int)((w >> 12) & 0xFFFu), band = (int)(w >> 24); // NONE: band 255
+                        if (band < nbands && row >= row_lo && row < row_hi && col + VK > col_lo && col < col_hi) {
+                            const T *q = reinterpret_cast<const T *>(base + gbyte[i]);
+                            if (col >= col_lo && col + VK <= col_hi) {
+                                __builtin_memcpy(&v, q, sizeof(vec));
+                            } else {
+#pragma unroll
+                                for (int e = 0; e < VK; ++e)
+                                    if (col + e >= col_lo && col + e < col_hi) v[e] = q[e];
+                            }
+                        }
+                    }
+                    val[j] = v;
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < BATCH; ++j) {
+                const int i = i0 + j;
+                if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) *reinterpret_cast<vec *>(lds + lds_at[i]) = val[j];
+            }
+        }
+    }
+};
+
 // Wavefront `wave`'s share of one staged stage: column chunks [kc_lo, kc_hi) x left rows [row0, row0 + nrows).
 template <class C>
 __device__ __forceinline__ void mfma_stage(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
@@ -238,6 +319,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
     // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner). (Fetching the next stage into
     // registers before the current one is swept, to hide the load latency behind the matrix instructions, measured
     // 2 % slower on large matrices and no faster on small ones: the other blocks of the CU already cover it.)
+    BandStager<C, C::NVB, C::RL, C::PV, C::PV, C::VBAND> left_stager;
+    BandStager<C, C::NUB, C::RU, C::KBX, C::PU, C::UBAND> right_stager; // (the padding columns of a right row are never read)
+    left_stager.init(tid, W, HW);
+    right_stager.init(tid, W, HW);
+    const T *left_first = g.V + (size_t)v_first * HW, *right_first = g.U + (size_t)u_first * HW;
     for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
             __syncthreads(); // everyone is done reading the previous stage
@@ -252,10 +338,8 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
                 const int ur_lo = yr0 < 0 ? -yr0 : 0;
                 const int ur_hi = H - yr0 < C::RU ? H - yr0 : C::RU;
                 const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
-                stage_bands<C, C::NVB, C::NVB, C::RL, C::PV, C::VBAND>(Vs, g.V + (size_t)v_first * HW, HW, 0, W, nbv, 1, 0, rows_ok, yl0, xbase, vc_lo,
-                                                                       vc_hi, tid);
-                stage_bands<C, C::NUB, C::NUL, C::RU, C::PU, C::UBAND>(Us, g.U + (size_t)u_first * HW, HW, 0, W, nbu, 1, ur_lo, ur_hi, yr0, x0, 0,
-                                                                       uc_hi, tid);
+                left_stager.stage(Vs, left_first + (ptrdiff_t)yl0 * W + xbase, nbv, 0, rows_ok, vc_lo, vc_hi);
+                right_stager.stage(Us, right_first + (ptrdiff_t)yr0 * W + x0, nbu, ur_lo, ur_hi, 0, uc_hi);
             }
             __syncthreads();
             // left rows of this stage that can overlap the tile's y shifts: yl in [syb, syb + TYB - 1 + H - 1], yl < chi
