@@ -71,7 +71,7 @@ static const EngineSpec specs[] = {
     make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.727, 6.347),
     make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8", 0.956, 5.555),
     make_spec<Z_84_u8>("f32_a8b4_lr8", 0.64, 6.951),
-    make_spec<Z_84_v4u8>("f32_a8b4_ll4lr8", 0.78, 0.973),
+    make_spec<Z_84_v4u8>("f32_a8b4_ll4lr8", 0.90, 0.973),
     make_spec<Z_44_u4>("f32_a4b4_lr4", 0.86, 2.5),
     make_spec<Z_44_u8>("f32_a4b4_lr8", 0.87, 2.5),
     make_spec<N_1x1>("f32_a1b4"),

@@ -253,16 +253,31 @@ __device__ __forceinline__ void mfma_stage(const typename C::value_type *Vs_lane
         j_last = (last - 1) % nrows + 1;
     }
     for (int kc = kc_a; kc < kc_b; kc += kc_step) {
-        const int ja = kc == kc_a ? j_first : 0;
-        const int jb = kc + kc_step >= kc_b ? j_last : nrows;
+        // (wavefront-uniform by construction; said so that the loop below is counted in scalar registers)
+        const int ja = __builtin_amdgcn_readfirstlane(kc == kc_a ? j_first : 0);
+        const int jb = __builtin_amdgcn_readfirstlane(kc + kc_step >= kc_b ? j_last : nrows);
         const T *vp = Vs_lane + kc * C::K + (row0 + ja) * C::PV;
         const T *up = Us_lane + kc * C::K + (row0 + ja) * C::PU;
         // two operand sets: the reads of the next row are issued before the instructions of the current one (the read
-        // past the last row of a sweep lands in the spare row the bands end with and is not used)
+        // past the last row of a sweep lands in the spare row the bands end with and is not used); four rows per trip
+        // so that the addresses advance once per sixteen-plus instructions
         evec a0[C::TI], a1[C::TI];
         T b0[C::TJ][EV], b1[C::TJ][EV];
         load(vp, up, a0, b0);
         int j = ja;
+#pragma unroll 1
+        for (; j + 4 <= jb; j += 4) {
+            load(vp + C::PV, up + C::PU, a1, b1);
+            multiply(a0, b0);
+            load(vp + 2 * C::PV, up + 2 * C::PU, a0, b0);
+            multiply(a1, b1);
+            load(vp + 3 * C::PV, up + 3 * C::PU, a1, b1);
+            multiply(a0, b0);
+            vp += 4 * C::PV;
+            up += 4 * C::PU;
+            load(vp, up, a0, b0);
+            multiply(a1, b1);
+        }
 #pragma unroll 1
         for (; j + 2 <= jb; j += 2) {
             load(vp + C::PV, up + C::PU, a1, b1);
