@@ -56,7 +56,10 @@ constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 
 // NC_: accumulator sets per result tile. The VK instructions of a step that feed one result tile form a dependent chain;
 // with NC_ > 1 they alternate between NC_ sets that are added up at the end, so a wavefront with few result tiles still
 // has independent instructions in flight (measured on the one-tile fp32 sweep: 0.89 -> 0.96 of the instruction's peak).
-template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int NC_ = 1, int WZ_ = 4, int SB_ = 8>
+// AL_ = 1: the left bands start on a 128-bit boundary of the matrix rows (see mfma_kernel); costs up to VK - 1 more columns per
+// left row, saves the element-wise assembly of pieces at the matrix edges: for tiles that mostly run on small matrices.
+template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int AL_ = 0, int NC_ = 1, int WZ_ = 4,
+          int SB_ = 8>
 struct MfmaCfg {
     using value_type = T;
     using Op = MfmaOp<T>;
@@ -71,7 +74,7 @@ struct MfmaCfg {
     static constexpr int TXB = JX * MJX, TYB = IY * NIY, TXW = TXB, TYW = TYB;
     static constexpr int NVB = JV * MJV, NUL = IU * NIU, NUB = NUL;
     static constexpr int WX = 1, WY = 1, WZ = WZ_, NWAVES = WZ, NT = 64 * NWAVES;
-    static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_;
+    static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_, AL = AL_;
     // what the launch record and the planner call the tile: shifts and matrices per lane, lanes over each
     static constexpr int A = (1 << popcount_c(Op::REG_BITS & (IY - 1))) * NIY;
     static constexpr int B = MJX;
@@ -81,7 +84,8 @@ struct MfmaCfg {
     static constexpr int LY = 1 << popcount_c(Op::LANE_BITS & (IY - 1));
     static constexpr int LU = 1 << popcount_c(Op::LANE_BITS & ~(IY - 1));
     // LDS geometry (elements). Left band: RL rows of every column a shift of the tile can meet in a stage.
-    static constexpr int PV = (TXB + KBX - 1 + VK - 1) / VK * VK;
+    // (+ VK - 1: the band starts at the 128-bit boundary of the matrix row at or below its first column, see mfma_kernel)
+    static constexpr int PV = (TXB + KBX - 1 + (AL ? VK - 1 : 0) + VK - 1) / VK * VK;
     // Lanes p = 0 .. P-1 read element (left matrix p / JX, column p % JX) of one row with one instruction: with the bands
     // JX (modulo the 256 bytes of the banks) apart they fall on P consecutive banks like the lanes of a single matrix.
     static constexpr int BANK_ELEMS = 256 / (int)sizeof(T);
@@ -174,6 +178,9 @@ struct BandStager {
                     if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) __builtin_memcpy(&val[j], base + gbyte[i], sizeof(vec)); // element-aligned only
                 }
             } else {
+                // pieces that straddle a column bound exist only where a bound is not a multiple of VK (matrices whose
+                // width is not; the stage origins themselves are kept on 128-bit boundaries)
+                const bool ragged = col_lo % VK != 0 || col_hi % VK != 0;
 #pragma unroll
                 for (int j = 0; j < BATCH; ++j) {
                     const int i = i0 + j;
@@ -183,15 +190,13 @@ struct BandStager {
                     if (i < ITER) {
                         const unsigned w = where[i];
                         const int col = (int)(w & 0xFFFu), row = (int)((w >> 12) & 0xFFFu), band = (int)(w >> 24); // NONE: band 255
-                        if (band < nbands && row >= row_lo && row < row_hi && col + VK > col_lo && col < col_hi) {
-                            const T *q = reinterpret_cast<const T *>(base + gbyte[i]);
-                            if (col >= col_lo && col + VK <= col_hi) {
-                                __builtin_memcpy(&v, q, sizeof(vec));
-                            } else {
+                        const bool in_rows = band < nbands && row >= row_lo && row < row_hi;
+                        const T *q = reinterpret_cast<const T *>(base + gbyte[i]);
+                        if (in_rows && col >= col_lo && col + VK <= col_hi) __builtin_memcpy(&v, q, sizeof(vec));
+                        if (ragged && in_rows && (col < col_lo || col + VK > col_hi) && col + VK > col_lo && col < col_hi) {
 #pragma unroll
-                                for (int e = 0; e < VK; ++e)
-                                    if (col + e >= col_lo && col + e < col_hi) v[e] = q[e];
-                            }
+                            for (int e = 0; e < VK; ++e)
+                                if (col + e >= col_lo && col + e < col_hi) v[e] = q[e];
                         }
                     }
                     val[j] = v;
@@ -314,7 +319,11 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
     const int p = lane % P, kk = lane / P;
     const int vj = p / C::JX, sxl = p % C::JX; // column j = p: left matrix, x shift
     const int ui = p / C::IY, syl = p % C::IY; // row i = p: right matrix, y shift
-    const T *Vs_lane = Vs + vj * C::VBAND + sxl + C::EV * kk;
+    // With AL the left bands start at the 128-bit boundary of the matrix rows at or below the tile's first column (x0 is a multiple of
+    // 8): every staged piece is then aligned in global memory and, where the width is a multiple of VK, wholly inside or
+    // outside the matrix; the lanes read `left_shift` columns further in.
+    const int left_shift = C::AL ? ((sxb % VK) + VK) % VK : 0;
+    const T *Vs_lane = Vs + vj * C::VBAND + sxl + C::EV * kk + left_shift;
     const T *Us_lane = Us + ui * C::UBAND + (C::TYB - 1 - syl) * C::PU + C::EV * kk;
 
     acc_t acc[C::TJ][C::TI][C::NC];
@@ -343,15 +352,15 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
             __syncthreads(); // everyone is done reading the previous stage
             {
-                // left band: rows [yl0, yl0+RL), columns xl = x0 + sxb + col
-                const int xbase = x0 + sxb;
-                const int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
-                const int vc_lo = xbase < 0 ? -xbase : 0;
-                const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
+                // left band: rows [yl0, yl0+RL), columns xl = x0 + sxb - shift + col (the 128-bit boundary at or below x0 + sxb)
+                const int xbase = x0 + sxb - left_shift;
                 // right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col
                 const int yr0 = yl0 - syb - C::TYB + 1;
                 const int ur_lo = yr0 < 0 ? -yr0 : 0;
                 const int ur_hi = H - yr0 < C::RU ? H - yr0 : C::RU;
+                const int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
+                const int vc_lo = xbase < 0 ? -xbase : 0;
+                const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
                 const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
                 left_stager.stage(Vs, left_first + (ptrdiff_t)yl0 * W + xbase, nbv, 0, rows_ok, vc_lo, vc_hi);
                 right_stager.stage(Us, right_first + (ptrdiff_t)yr0 * W + x0, nbu, ur_lo, ur_hi, 0, uc_hi);

@@ -6,7 +6,7 @@
 
 namespace xcorr {
 
-//                              T   JV IU MJX MJV NIY NIU  RL KBX MINB
+//                              T   JV IU MJX MJV NIY NIU  RL KBX MINB AL
 // one pair per block
 using M_32x32 = MfmaCfg<float, 1, 1, 1, 1, 1, 1, 32, 64, 4>;
 using M_64x32 = MfmaCfg<float, 1, 1, 2, 1, 1, 1, 32, 64, 4>;
@@ -14,7 +14,7 @@ using M_64x32 = MfmaCfg<float, 1, 1, 2, 1, 1, 1, 32, 64, 4>;
 using M_32x8_r4 = MfmaCfg<float, 1, 4, 1, 1, 1, 1, 32, 32, 4>;
 using M_32x8_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 32, 32, 3>;
 // ... and rows over right, columns over left matrices (n_to_m)
-using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 32, 32, 3>;
+using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 32, 32, 3, 1>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)

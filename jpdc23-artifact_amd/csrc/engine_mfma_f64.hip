@@ -6,11 +6,11 @@
 
 namespace xcorr {
 
-//                               T    JV IU MJX MJV NIY NIU  RL KBX MINB
+//                               T    JV IU MJX MJV NIY NIU  RL KBX MINB AL
 using D_32x32 = MfmaCfg<double, 1, 1, 2, 1, 2, 1, 32, 32, 4>;
 using D_32x16 = MfmaCfg<double, 1, 1, 2, 1, 1, 1, 32, 32, 4>;
 using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
-using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 16, 32, 3>;
+using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 16, 32, 3, 1>;
 
 static const EngineSpec specs[] = {
     make_spec<D_32x32>("f64_m32x32", 0.75, 1.0),
