@@ -226,9 +226,13 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         const bool matrices_in_tile = s.MFMA ? s.NVB() * s.NUB() > 1 : s.LV * s.LU > 1;
         for (int k : ladder) {
             int rc = k * G;
-            if (rq.rows_per_worker > 0 || rq.caller_zeroes) {
+            if (rq.rows_per_worker > 0) {
                 if (k != 0) break;
                 rc = (int)rq.rows_per_worker;
+            } else if (rq.caller_zeroes) {
+                // zeroed output, atomic adds, no chunk named: whole rows (k = 0) or any chunk of the ladder
+                if (k == 0) rc = rq.H;
+                if (k != 0 && (rc >= rq.H || rq.dist == XCORR_DIST_NONE)) break;
             } else if (k != 0 && (!rq.may_split || rc >= rq.H)) {
                 break;
             } else if (k != 0 && matrices_in_tile && (rc < 36 || rq.H < 72)) {
@@ -274,6 +278,31 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
                     specs[rq.spec_index - 1].name);
     const bool grouped = rq.spec_index > 0 ? specs[rq.spec_index - 1].A > 1 : rq.y_shifts != 1;
     if (grouped) return plan_grouped(rq, specs, count, plan);
+
+    // The one-output-row families are contracts (who clears the output, how the rows are dealt to workers), not kernels:
+    // where the caller names no tile geometry, a matrix-core tile serves them under the same contract (its work items
+    // take the caller's rows per worker and distribution like any other tile's). Measured against the one-row tiles
+    // (fp32, 16x16 ... 1024x1024, 1 ... 1024 pairs): 1.2-4.9x faster from 64x64 on and from eight pairs of 32x32 on,
+    // 0.8-1.0x below; taken from 8192 elements per launch on (pairs x rows x columns), for a single pair from 64x64 on.
+    const bool no_tile_asked = rq.spec_index == 0 && rq.x_shifts == 0 && rq.lanes_x == 0 && rq.lanes_y == 0 && rq.left_mats <= 1 && rq.right_mats <= 1;
+    const double pair_count = rq.group_m > 0 ? (double)rq.nU : (double)rq.nV * rq.nU;
+    const double elements = pair_count * rq.W * rq.H;
+    const bool large_enough = pair_count >= 2.0 ? elements >= 8192.0 : (double)rq.W * rq.H >= 4096.0;
+    // (a caller who fixes short chunks of rows wants the reference's work distribution: left to the one-row tiles)
+    const bool chunk_fits = rq.rows_per_worker == 0 || rq.rows_per_worker >= 16 || rq.dist == XCORR_DIST_NONE; // ("none": the chunk is not used)
+    // (a plain launcher told to keep the rows whole promises the summation order of one pass over the rows, which is what
+    // brings the large fp32 pair within 1e-5 of the reference's fp32 host loop: the one-row tiles keep it)
+    const bool order_free = rq.may_split || rq.caller_zeroes;
+    if (no_tile_asked && (rq.matrix_cores == 1 || (rq.matrix_cores == 0 && large_enough && chunk_fits && order_free))) {
+        EngineRequest q = rq;
+        q.y_shifts = q.left_mats = q.right_mats = 0;
+        q.matrix_cores = 1;
+        // (no distribution named: chunks of one tile follow each other, "triangle"; the reference's default, "rectangle",
+        // interleaves the tiles and was measured up to 2x slower with these tiles - blocks that run together then stage
+        // rows far apart)
+        if (q.caller_zeroes && q.dist == XCORR_DIST_DEFAULT) q.dist = XCORR_DIST_TRIANGLE;
+        return plan_grouped(q, specs, count, plan);
+    }
 
     // one-output-row families: relative cost of the tile, then the split rule below
     const EngineSpec *best = rq.spec_index > 0 ? &specs[rq.spec_index - 1] : nullptr;

@@ -31,7 +31,13 @@ def plan():
         lib.xcorr_plan_only(0)
 
 
+def register_tiles(plan):
+    """The same planner with the matrix-core tiles excluded: the rules of the one-output-row tiles."""
+    return lambda *a, **kw: plan(*a, matrix_cores=2, **kw)
+
+
 def test_plain_one_row_launcher_splits_only_when_it_pays(plan):
+    plan = register_tiles(plan)
     rec = plan("shuffle", 64, 64)
     assert rec["kernel"] == "shuffle/f32_a1b4" and rec["uses_atomics"] == 1 and 3 <= rec["rows_per_worker"] <= 8
     rec = plan("shuffle", 64, 64, distribution_type="none")
@@ -45,6 +51,7 @@ def test_plain_one_row_launcher_splits_only_when_it_pays(plan):
 
 
 def test_split_row_chunk(plan):
+    plan = register_tiles(plan)
     # the caller's chunk and distribution are taken as given
     rec = plan("split_row", 100, 90, rows_per_thread=7, distribution_type="triangle")
     assert rec["rows_per_worker"] == 7 and rec["distribution_type"] == 3 and rec["uses_atomics"] == 1
@@ -61,6 +68,7 @@ def test_split_row_chunk(plan):
 
 
 def test_matrices_per_lane(plan):
+    plan = register_tiles(plan)
     # small launches: one matrix per lane; a request for matrices per thread overrides; large launches reuse
     assert plan("multimat_both", 16, 16, 2, 2)["kernel"] == "multimat_both/f32_a1b4"
     assert plan("multimat_both", 16, 16, 2, 2, right_matrices_per_thread=4)["kernel"] == "multimat_both/f32_a1b4_r4"
@@ -123,8 +131,28 @@ def test_matrix_core_tiles(plan):
     xc = load_package()
     with pytest.raises(xc.XcorrError, match="matrix_cores must be 0, 1 or 2"):
         plan("grouped_overlap", 300, 300, matrix_cores=3)
-    # the one-output-row families have no matrix-core tiles
-    assert plan("split_row", 256, 256)["matrix_cores"] == 0
+
+
+def test_one_row_families_on_matrix_core_tiles(plan):
+    """The one-output-row families are contracts: large enough launches that name no tile run a matrix-core tile under them."""
+    rec = plan("split_row", 256, 256)
+    assert rec["matrix_cores"] == 1 and rec["kernel"].startswith("split_row/f32_m") and rec["uses_atomics"] == 1 and rec["distribution_type"] == 3
+    rec = plan("split_row", 256, 256, rows_per_thread=32, distribution_type="rectangle")
+    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 32 and rec["distribution_type"] == 2
+    rec = plan("split_row", 256, 256, distribution_type="none")
+    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 256 and rec["uses_atomics"] == 1
+    # short chunks of rows fixed by the caller, a tile request, small launches, matrix_cores = 2: the one-row tiles
+    assert plan("split_row", 256, 256, rows_per_thread=7)["matrix_cores"] == 0
+    assert plan("multimat_right", 128, 128, 1, 32, right_matrices_per_thread=4)["matrix_cores"] == 0
+    assert plan("shuffle", 32, 32)["matrix_cores"] == 0 and plan("shuffle", 64, 64)["matrix_cores"] == 1
+    assert plan("multimat_both", 32, 32, 2, 2)["matrix_cores"] == 0 and plan("multimat_both", 32, 32, 8, 8)["matrix_cores"] == 1
+    assert plan("multimat_right", 32, 32, 1, 2)["matrix_cores"] == 0 and plan("multimat_right", 32, 32, 1, 32)["matrix_cores"] == 1
+    assert plan("multimat_right", 256, 256, 1, 32, matrix_cores=2)["matrix_cores"] == 0
+    # the plain launcher told to keep the rows whole keeps the summation order of one pass over the rows: a one-row tile
+    rec = plan("shuffle", 256, 256, distribution_type="none")
+    assert rec["matrix_cores"] == 0 and rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 256
+    # matrix_cores = 1 forces the route also for small launches
+    assert plan("shuffle", 16, 16, matrix_cores=1)["matrix_cores"] == 1
 
 
 def test_errors_in_plan_only_mode(plan):
