@@ -115,9 +115,11 @@ typedef struct xcorr_params {
     unsigned whole_pair_in_lds;              /* grouped-overlap, one small pair: 0 = the launcher decides, 1 = always run the kernel that
                                                 keeps both matrices in LDS (an error if they do not fit), 2 = never; no counterpart
                                                 in the reference */
-    unsigned matrix_cores;                   /* grouped engine families: 0 = the launcher decides between its register tiles (vector FMA) and
-                                                its matrix-core tiles (v_mfma), 1 = matrix-core tiles only, 2 = never; no counterpart in
-                                                the reference */
+    unsigned matrix_cores;                   /* engine families: 0 = the launcher decides between its register tiles (vector FMA) and
+                                                its matrix-core tiles (v_mfma), 1 = matrix-core tiles only, 2 = never; the one-output-row
+                                                launchers (shuffle, split_row, multimat_right, multimat_both) take a matrix-core tile
+                                                under their own contract when no tile geometry and no chunk below 16 rows is named
+                                                and the launch is large enough; no counterpart in the reference */
 } xcorr_params;
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the

@@ -67,8 +67,8 @@ static const EngineSpec specs[] = {
     make_spec<Z_88_u4>("f32_a8b8_lr4", 0.692, 10.581),
     make_spec<Z_84_u16>("f32_a8b4_lr16", 0.82, 4.421),
     make_spec<Z_88_u16>("f32_a8b8_lr16", 0.76, 8.433),
-    make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4", 0.811, 0.973),
-    make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.727, 6.347),
+    make_spec<Z_84_v4u4>("f32_a8b4_ll4lr4", 0.875, 0.973),
+    make_spec<Z_88_v4u4>("f32_a8b8_ll4lr4", 0.78, 6.347),
     make_spec<Z_88_v8u8>("f32_a8b8_ll8lr8", 0.956, 5.555),
     make_spec<Z_84_u8>("f32_a8b4_lr8", 0.64, 6.951),
     make_spec<Z_84_v4u8>("f32_a8b4_ll4lr8", 0.90, 0.973),

@@ -45,7 +45,7 @@ static const EngineSpec specs[] = {
     make_spec<Z_88_v8u8>("f64_a8b8_ll8lr8", 0.637, 12.851),
     make_spec<Y_84_u4>("f64_a8b4_lr4", 0.733, 0.0),
     make_spec<Y_84>("f64_a8b4", 0.676, 0.0),
-    make_spec<D_84_v4u4>("f64_a8b4_ll4lr4", 0.768, 0.0),
+    make_spec<D_84_v4u4>("f64_a8b4_ll4lr4", 0.81, 0.0),
     make_spec<D_84_v4u8>("f64_a8b4_ll4lr8", 0.84, 0.0),
     make_spec<Z_44_u4>("f64_a4b4_lr4", 0.82, 1.0),
     make_spec<Z_44_u8>("f64_a4b4_lr8", 0.85, 1.0),

@@ -22,7 +22,7 @@ static const EngineSpec specs[] = {
     make_spec<M_64x32>("f32_m64x32", 0.82, 1.0),
     make_spec<M_32x8_r4>("f32_m32x8_r4", 0.82, 1.0),
     make_spec<M_32x8_r8>("f32_m32x8_r8", 0.88, 1.0),
-    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 1.0, 1.0),
+    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.96, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f32(int *count) {

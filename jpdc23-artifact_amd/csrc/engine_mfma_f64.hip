@@ -16,7 +16,7 @@ static const EngineSpec specs[] = {
     make_spec<D_32x32>("f64_m32x32", 0.75, 1.0),
     make_spec<D_32x16>("f64_m32x16", 0.80, 1.0),
     make_spec<D_32x8_r4>("f64_m32x8_r4", 0.78, 1.0),
-    make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.95, 1.0),
+    make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.92, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f64(int *count) {
