@@ -202,11 +202,23 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
     static const int ladder[] = {0, 2, 3, 4, 6, 8, 12, 16, 24, 32};
     bool found = false;
     double best = 0;
+    int candidate_error = XCORR_OK;
     RequestMatch best_match = {};
     for (int i = 0; i < count; ++i) {
         const EngineSpec &s = specs[i];
         if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
         if (rq.group_m > 0 ? (s.NVB() != 1 && !s.PG) : s.PG != 0) continue; // lanes over left matrices: all pairs, or paired groups
+        // A matrix-core tile addresses the pieces it stages by 32-bit byte offsets from the first matrix of its block: its
+        // bands must lie within 4 GiB of each other (they always do for one matrix per block; tiles of several matrices are
+        // for small matrices anyway).
+        const int bands = s.NVB() > s.NUB() ? s.NVB() : s.NUB();
+        const bool offsets_fit = !s.MFMA || bands == 1 || (double)bands * rq.W * rq.H * s.elem_bytes < 4.0e9;
+        if (!offsets_fit) {
+            if (rq.spec_index > 0)
+                return fail(XCORR_ERR_UNSUPPORTED, "%s: specialisation %s stages %d matrices per block through 32-bit offsets; %d x %d matrices are too large for it",
+                            rq.family, s.name, bands, rq.H, rq.W);
+            continue;
+        }
         if (rq.spec_index == 0) {
             if (rq.matrix_cores == 1 ? !s.MFMA : rq.matrix_cores == 2 ? s.MFMA != 0 : false) continue;
             if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
@@ -239,7 +251,11 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
                 continue; // measured: short chunks of tiles whose lanes lie over matrices lose to their scattered atomic adds
             }
             EnginePlan cand;
-            if (int e = shape_plan(s, rq, rc, (int)rq.column_chunks, cand)) return e;
+            if (int e = shape_plan(s, rq, rc, (int)rq.column_chunks, cand)) {
+                // (more work items than the launch arithmetic holds, e.g. short chunks of a 16384x16384 pair: another candidate will do)
+                candidate_error = e;
+                continue;
+            }
             const double t = predict_us(s, rq, cand);
             if (!found || match.better_than(best_match) || t < best) {
                 found = true;
@@ -250,6 +266,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
             }
         }
     }
+    if (!found && candidate_error != XCORR_OK) return candidate_error; // (its message is the last error text)
     if (!found)
         return fail(XCORR_ERR_UNSUPPORTED, "%s: no compiled specialisation matches x_shifts_per_thread=%u lanes_x=%u lanes_y=%u",
                     rq.family, rq.x_shifts, rq.lanes_x, rq.lanes_y);
@@ -283,11 +300,14 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     // where the caller names no tile geometry, a matrix-core tile serves them under the same contract (its work items
     // take the caller's rows per worker and distribution like any other tile's). Measured against the one-row tiles
     // (fp32, 16x16 ... 1024x1024, 1 ... 1024 pairs): 1.2-4.9x faster from 64x64 on and from eight pairs of 32x32 on,
-    // 0.8-1.0x below; taken from 8192 elements per launch on (pairs x rows x columns), for a single pair from 64x64 on.
+    // 0.8-1.0x below; taken from 8192 elements per launch on (pairs x rows x columns), for a single pair from 64x64 on
+    // (fp64: from 32x32 matrices on).
     const bool no_tile_asked = rq.spec_index == 0 && rq.x_shifts == 0 && rq.lanes_x == 0 && rq.lanes_y == 0 && rq.left_mats <= 1 && rq.right_mats <= 1;
     const double pair_count = rq.group_m > 0 ? (double)rq.nU : (double)rq.nV * rq.nU;
     const double elements = pair_count * rq.W * rq.H;
-    const bool large_enough = pair_count >= 2.0 ? elements >= 8192.0 : (double)rq.W * rq.H >= 4096.0;
+    const double area = (double)rq.W * rq.H;
+    // (fp64: measured 1.1-1.5x faster already on 32x32 matrices, 1.5-5.4x beyond)
+    const bool large_enough = rq.elem_bytes == 8 ? area >= 1024.0 : pair_count >= 2.0 ? elements >= 8192.0 : area >= 4096.0;
     // (a caller who fixes short chunks of rows wants the reference's work distribution: left to the one-row tiles)
     const bool chunk_fits = rq.rows_per_worker == 0 || rq.rows_per_worker >= 16 || rq.dist == XCORR_DIST_NONE; // ("none": the chunk is not used)
     // (a plain launcher told to keep the rows whole promises the summation order of one pass over the rows, which is what
@@ -313,8 +333,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     // measured (fp32, 1 x 8 ... 1 x 256 and 2 x 2 ... 32 x 32 matrices of 16x16 ... 256x256) the one-matrix tiles win up to
     // about 3e9 multiply-adds per launch (by 1.2-1.5x on the smallest), the others beyond; a request for matrices per
     // thread overrides this.
-    const double pairs = rq.group_m > 0 ? (double)rq.nU : (double)rq.nV * rq.nU;
-    const double area = (double)rq.W * rq.H;
+    const double pairs = pair_count;
     const bool one_matrix_per_lane = rq.left_mats <= 1 && rq.right_mats == 0 && pairs * area * area < 3e9;
     for (int i = 0; i < count && rq.spec_index == 0; ++i) {
         const EngineSpec &s = specs[i];

@@ -156,6 +156,18 @@ def test_one_row_families_on_matrix_core_tiles(plan):
     assert plan("shuffle", 16, 16, matrix_cores=1)["matrix_cores"] == 1
 
 
+def test_largest_matrices(plan):
+    # 16384 x 16384: chunk sizes whose work items do not fit the launch arithmetic are passed over, not reported
+    rec = plan("grouped_overlap", 16384, 16384)
+    assert rec["grid"][0] > 0 and rec["matrix_cores"] == 1
+    # tiles that stage several matrices per block address them through 32-bit offsets: left out where 4 GiB do not hold them
+    rec = plan("multimat_right_grouped", 16384, 16384, 1, 8)
+    assert rec["right_matrices_per_thread"] * rec["lanes_right"] == 1
+    xc = load_package()
+    with pytest.raises(xc.XcorrError, match="32-bit offsets"):
+        plan("multimat_right_grouped", 16384, 16384, 1, 8, specialisation=25)
+
+
 def test_errors_in_plan_only_mode(plan):
     xc = load_package()
     with pytest.raises(xc.XcorrError, match="Too many shifts per thread: 9"):
