@@ -115,3 +115,47 @@ def test_never_and_only(oracle):
         assert np.array_equal(got, exp)
     with pytest.raises(xc.XcorrError, match="matrix_cores must be 0, 1 or 2"):
         xc.run("grouped_overlap", left, right, 1, params=xc.make_params(matrix_cores=7))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_one_output_row_families_on_matrix_core_tiles(oracle, dtype):
+    """shuffle, split_row, multimat_right(_groups) and multimat_both served by matrix-core tiles under their own contracts
+    (who clears the output, rows per worker, distribution): forced with matrix_cores = 1 on small shapes, chosen by the
+    launcher on larger ones."""
+    xc = load_package()
+    rng = np.random.default_rng(904)
+    seen = set()
+    contracts = [{}, dict(rows_per_thread=16), dict(rows_per_thread=40, distribution_type="rectangle"), dict(distribution_type="triangle"),
+                 dict(distribution_type="none")]
+    for shape in [(5, 3), (31, 33), (64, 64), (70, 130)]:
+        left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
+        exp = oracle.one_to_one(left, right, threads=4)
+        for family in ("shuffle", "split_row"):
+            for kw in contracts:
+                if family == "shuffle" and "rows_per_thread" in kw:
+                    continue
+                say(family, np.dtype(dtype).name, shape, kw)
+                launch_and_check(xc, family, left, right, 1, 1, 1, exp, True, kw, seen)
+        for n_right in (3, 9):
+            many = ints(rng, (n_right,) + shape, dtype)
+            exp_many = oracle.one_to_many(left[None], many)
+            for kw in contracts:
+                say("multimat_right", np.dtype(dtype).name, shape, n_right, kw)
+                launch_and_check(xc, "multimat_right", left[None], many, n_right, 1, n_right, exp_many, True, kw, seen)
+        lefts, rights = ints(rng, (3,) + shape, dtype), ints(rng, (6,) + shape, dtype)
+        exp_groups = np.concatenate([oracle.one_to_many(lefts[l:l + 1], rights[2 * l:2 * l + 2]) for l in range(3)])
+        exp_all = oracle.n_to_m(lefts, rights, threads=4)
+        for kw in contracts[:4]:
+            say("multimat_right_groups / multimat_both", np.dtype(dtype).name, shape, kw)
+            launch_and_check(xc, "multimat_right_groups", lefts, rights, 6, 3, 2, exp_groups, True, kw, seen)
+            launch_and_check(xc, "multimat_both", lefts, rights, 18, 3, 6, exp_all, True, kw, seen)
+    # the launcher's own choice on a launch that is large enough, and the cases it leaves to the one-row tiles
+    left, right = ints(rng, (150, 140), dtype), ints(rng, (150, 140), dtype)
+    exp = oracle.one_to_one(left, right, threads=4)
+    for family, kw, routed in [("split_row", {}, 1), ("shuffle", {}, 1), ("split_row", dict(rows_per_thread=7), 0), ("shuffle", dict(distribution_type="none"), 0),
+                               ("split_row", dict(matrix_cores=2), 0)]:
+        got = xc.run(family, left, right, 1, params=xc.make_params(**kw))
+        rec = xc.last_launch()
+        assert rec["matrix_cores"] == routed, (family, kw, rec["kernel"])
+        assert np.array_equal(got, exp), (family, kw, rec["kernel"])
+    say(sorted(seen))
