@@ -9,15 +9,19 @@
 // so the whole reduction over (yl, xr) accumulates into the same P x P result tile of v_mfma_f32_32x32x2_f32 (P = 32,
 // two k slots) or v_mfma_f64_16x16x4_f64 (P = 16, four k slots). Nothing is multiplied that the definition does not
 // multiply, except the zero padding at tile edges that the register-tile sweep has as well. Both instructions run at
-// the rate of the vector FMA peak, but one instruction keeps the pipeline busy for 64 / 32 cycles, so the LDS reads
-// and address arithmetic around it are free, and operand reuse happens inside the matrix core instead of in
-// registers: small shift tiles (many matrices per tile) cost nothing extra.
+// the rate of the vector FMA peak (64 cycles each on this chip), but one instruction stands for 2048 / 1024 FMAs: the
+// LDS reads and address arithmetic around it weigh little (about two cycles of the matrix pipeline per other
+// instruction issued on the SIMD), the shader clock stays at 2.35 GHz on data that holds the vector-FMA loop at 2.0-2.1,
+// and operand reuse happens inside the matrix core instead of in registers: small shift tiles (many matrices per tile)
+// cost nothing extra.
 //
 // Lane l of a wavefront (p = l % P, kk = l / P) supplies row i = p of Ua and column j = p of Vb for k slot kk. The k
 // slots of the EV instructions of a step (4 for the 32 x 32 fp32 tile, 2 for the 16 x 16 fp64 tile) are assigned
 // x_k = x0 + EV * kk + e, e = 0 .. EV-1, so the right operand of a step is ONE aligned LDS read of EV elements per lane
-// and the left operand EV consecutive elements. A step covers 8 right columns with every instruction. The LDS bands, their staging, the work items and the split of a
-// stage's column chunks over the four wavefronts of a block are those of the register-tile sweep (engine.hpp).
+// and the left operand EV consecutive elements. A step covers 8 right columns with every instruction. The work items
+// (tiles, chunks of rows and columns, centre-out order), the zero-padded LDS bands and the four wavefronts of a block
+// that share one tile are those of the register-tile sweep (engine.hpp); the staging (BandStager) and the deal of a
+// stage's steps to the wavefronts (mfma_stage) are this file's.
 //
 // Result layout of the instructions (lane l, accumulator element r): column j = l % P; row i = 8 * (r / 4) + 4 * (l / 32) + r % 4
 // for the fp32 instruction and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs.
