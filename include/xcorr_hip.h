@@ -274,7 +274,7 @@ int xcorr_split_row_f64(const double *left, const double *right, double *out, un
  * Replaces run_ccn_shuffle_multirow_both (kernels.cuh:185-195). One pair.
  * `out` need not be zeroed: when the launcher splits the reduction to fill the
  * device it clears `out` itself on `stream` first. A pair small enough for both
- * matrices to sit in the LDS of one CU (run by default up to 112 x 112 fp32, 96 x 96 fp64) and given no tile
+ * matrices to sit in the LDS of one CU (run by default up to 96 x 96 fp32, 64 x 64 fp64) and given no tile
  * selection runs a kernel of its own kind instead: every block keeps the whole pair
  * in LDS and its wavefronts reduce groups of four adjacent x shifts, one launch,
  * no atomics (the role of run_ccn_warp_per_shift_shared_mem, kernels.cuh:144-161, at

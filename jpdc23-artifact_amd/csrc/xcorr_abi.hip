@@ -274,13 +274,14 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     if ((rc = check_dist(p.distribution_type))) return rc;
     if (p.whole_pair_in_lds > 2) return fail(XCORR_ERR_INVALID_ARGUMENT, "whole_pair_in_lds must be 0, 1 or 2, not %u", p.whole_pair_in_lds);
     // A small pair with no tile asked for: both matrices in the LDS of every block, one launch, no atomics. Measured
-    // against the engine's best plan on square pairs (microseconds per launch, whole-pair kernel / engine): fp32 16: 3.6 / 5.6,
-    // 32: 3.9 / 7.4, 64: 6.0 / 10.4, 80: 11.2 / 12.6, 96: 14.1 / 16.1, 112: 19.0 / 21.0, 128: 28.6 / 21.6; fp64 32: 4.4 / 8.0,
-    // 64: 8.6 / 13.1, 96: 19.2 / 23.3. Beyond the sizes below the engine's register tiles win.
+    // against the engine's best plan on square pairs (microseconds per launch, whole-pair kernel / engine, which runs a
+    // matrix-core tile from about 100x100 on): fp32 16: 3.9 / 5.3, 32: 4.1 / 7.3, 64: 5.5 / 10.3, 80: 11.9 / 12.3, 96: 12.5 / 13.7,
+    // 104: 15.4 / 14.1, 112: 18.4 / 14.8, 128: 28.4 / 17.3; fp64 32: 4.2 / 7.8, 64: 7.9 / 11.7, 72: 16.4 / 13.4, 96: 17.4 / 15.0.
+    // Beyond the sizes below the engine wins.
     const bool tile_asked = p.specialisation || p.x_shifts_per_thread || p.lanes_x || p.lanes_y || p.rows_per_thread || p.column_chunks ||
                             p.shifts_per_thread || p.matrix_cores || p.distribution_type != XCORR_DIST_DEFAULT;
     const size_t elems = (size_t)cols * rows;
-    const bool small = pair_fits_lds<T>(cols, rows) && cols <= 128 && elems <= (sizeof(T) == 4 ? 112u * 112u : 96u * 96u);
+    const bool small = pair_fits_lds<T>(cols, rows) && cols <= 128 && elems <= (sizeof(T) == 4 ? 96u * 96u : 64u * 64u);
     if (p.whole_pair_in_lds == 1 || (p.whole_pair_in_lds == 0 && !tile_asked && small))
         return run_pair_in_lds<T>("grouped_overlap", left, right, out, cols, rows, as_stream(stream));
     EngineRequest rq = base_request("grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);

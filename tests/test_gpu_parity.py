@@ -108,7 +108,7 @@ def test_one_to_one_all_families(oracle, dtype, family, kw):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_whole_pair_in_lds(oracle, dtype):
     """The kernel that keeps both matrices of a small pair in LDS (the default of grouped_overlap up to
-    112 x 112 fp32 / 96 x 96 fp64): every size 1 ... 12 squared, sizes around the 64-column chunk of its lanes,
+    96 x 96 fp32 / 64 x 64 fp64): every size 1 ... 12 squared, sizes around the 64-column chunk of its lanes,
     ragged non-square shapes and the largest pairs that fit; bit-exact on integers, within tolerance on real
     values; the launcher picks it by itself for small pairs and leaves larger ones to the engine; a pair that
     does not fit is an error when the kernel is forced."""
@@ -128,7 +128,8 @@ def test_whole_pair_in_lds(oracle, dtype):
         got = xc.run("grouped_overlap", left, right, 1, params=xc.make_params(whole_pair_in_lds=1))
         check(got, oracle.one_to_one(left, right), False, f"whole pair {shape} real")
     # the launcher's own choice
-    for shape, expect in [((64, 64), True), ((40, 90), True), ((110, 100), np.dtype(dtype) == np.float32), ((200, 200), False), ((3, 300), False)]:
+    for shape, expect in [((64, 64), True), ((40, 90), True), ((90, 100), np.dtype(dtype) == np.float32), ((110, 100), False),
+                          ((200, 200), False), ((3, 300), False)]:
         left, right = ints(rng, shape, dtype), ints(rng, shape, dtype)
         got = xc.run("grouped_overlap", left, right, 1)
         assert ("pair_in_lds" in xc.last_launch()["kernel"]) == expect, (shape, xc.last_launch()["kernel"])
