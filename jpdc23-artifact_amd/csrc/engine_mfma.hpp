@@ -60,10 +60,15 @@ constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 
 // NC_: accumulator sets per result tile. The VK instructions of a step that feed one result tile form a dependent chain;
 // with NC_ > 1 they alternate between NC_ sets that are added up at the end, so a wavefront with few result tiles still
 // has independent instructions in flight (measured on the one-tile fp32 sweep: 0.89 -> 0.96 of the instruction's peak).
+// JYO_: copies of the x shifts of a result tile's columns, IY left rows apart: column j <-> (copy c_j, x shift sx_j) reads
+// Vb[k][j] = V[yb + c_j * IY][x_k + sx_j] while row i reads U[yb - sy_i][x_k], so the tile holds the y shifts sy_i + c_j * IY:
+// P / JYO_ x shifts by IY * JYO_ y shifts of one left matrix instead of P by IY (a squarer tile sweeps fewer rows and columns that
+// only some of its shifts overlap). The copies come from the same LDS band, IY rows further down: they cost (JYO_ - 1) * IY
+// more rows per band and per chunk of left rows, no staging.
 // AL_ = 1: the left bands start on a 128-bit boundary of the matrix rows (see mfma_kernel); costs up to VK - 1 more columns per
 // left row, saves the element-wise assembly of pieces at the matrix edges: for tiles that mostly run on small matrices.
 template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int AL_ = 0, int NC_ = 1, int WZ_ = 4,
-          int SB_ = 8>
+          int SB_ = 8, int JYO_ = 1>
 struct MfmaCfg {
     using value_type = T;
     using Op = MfmaOp<T>;
@@ -72,12 +77,14 @@ struct MfmaCfg {
     static constexpr int VK = 16 / (int)sizeof(T);
     static constexpr int EV = Op::EV;   // consecutive elements a lane reads per operand and step = instructions per step and result tile
     static constexpr int K = KS * EV; // right columns per step (8)
-    static constexpr int JV = JV_, JX = P / JV_, IU = IU_, IY = P / IU_;
+    static constexpr int JV = JV_, JYO = JYO_, JX = P / (JV_ * JYO_), IU = IU_, IY = P / IU_;
     static constexpr int MJX = MJX_, MJV = MJV_, NIY = NIY_, NIU = NIU_;
     static constexpr int TJ = MJX * MJV, TI = NIY * NIU; // result tiles of a wavefront
-    static constexpr int TXB = JX * MJX, TYB = IY * NIY, TXW = TXB, TYW = TYB;
+    static constexpr int IYB = IY * NIY;                   // y shifts among the rows of the result tiles: the window of right rows of a left row
+    static constexpr int TXB = JX * MJX, TYB = IYB * JYO, TXW = TXB, TYW = IYB;
     static constexpr int NVB = JV * MJV, NUL = IU * NIU, NUB = NUL;
-    static constexpr int WX = 1, WY = 1, WZ = WZ_, NWAVES = WZ, NT = 64 * NWAVES;
+    // (the copies of the x shifts are reported as half or quarter wavefronts along y)
+    static constexpr int WX = 1, WY = JYO, WZ = WZ_, NWAVES = WZ, NT = 64 * NWAVES;
     static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_, AL = AL_;
     // what the launch record and the planner call the tile: shifts and matrices per lane, lanes over each
     static constexpr int A = (1 << popcount_c(Op::REG_BITS & (IY - 1))) * NIY;
@@ -89,23 +96,35 @@ struct MfmaCfg {
     static constexpr int LU = 1 << popcount_c(Op::LANE_BITS & ~(IY - 1));
     // LDS geometry (elements). Left band: RL rows of every column a shift of the tile can meet in a stage.
     // (+ VK - 1: the band starts at the 128-bit boundary of the matrix row at or below its first column, see mfma_kernel)
-    static constexpr int PV = (TXB + KBX - 1 + (AL ? VK - 1 : 0) + VK - 1) / VK * VK;
+    // The copies of the x shifts read rows IY apart with one instruction, P lanes a pass: with IY rows JX elements apart modulo
+    // the P x 4 bytes (fp64: P x 8) those lanes touch, they fall on P consecutive banks like the lanes of a single row (measured
+    // with IY rows a multiple of that apart: 0.35 conflict cycles per LDS cycle). No multiple of 128 bits does that for 8 rows:
+    // such a band keeps its rows on 64-bit boundaries only and is filled with 64-bit LDS stores.
+    static constexpr int BANK_ELEMS = 256 / (int)sizeof(T);
+    static constexpr int PVC = (TXB + KBX - 1 + (AL ? VK - 1 : 0) + VK - 1) / VK * VK; // columns of a left band
+    static constexpr int left_pitch() {
+        int n = PVC;
+        if (JYO > 1)
+            while ((IY * n) % (P * (int)sizeof(T) / 4) != JX || (n * (int)sizeof(T)) % 8 != 0) n += 1;
+        return n;
+    }
+    static constexpr int PV = left_pitch();
+    static constexpr int VROWS = RL + (JYO - 1) * IY; // rows of a left band
     // Lanes p = 0 .. P-1 read element (left matrix p / JX, column p % JX) of one row with one instruction: with the bands
     // JX (modulo the 256 bytes of the banks) apart they fall on P consecutive banks like the lanes of a single matrix.
-    static constexpr int BANK_ELEMS = 256 / (int)sizeof(T);
     static constexpr int left_band(int n) {
-        if (JV == 1) return n;
+        if (JV == 1) return (n + VK - 1) / VK * VK;
         int b = n;
         while (b % BANK_ELEMS != JX % BANK_ELEMS) b += VK;
         return b;
     }
-    static constexpr int VBAND = left_band((RL + 1) * PV); // one spare row: the sweep reads one row ahead
+    static constexpr int VBAND = left_band((VROWS + 1) * PV); // one spare row: the sweep reads one row ahead
     // Right band: an LDS pass serves the reads of 32 consecutive lanes, and the EV-element pieces they touch must differ
     // modulo 32 (measured: one collision doubles the pass). Those lanes are rows p = 0 .. P-1 apart and, for the 16-row
     // tiles, two k slots one piece apart: the row pitch is an odd number of pieces (P = 32) or twice an odd number
     // (P = 16), and the bands of the IU matrices of a result tile continue the row sequence (band stride = -IY rows
     // modulo 32 pieces).
-    static constexpr int RU = RL + TYB - 1;
+    static constexpr int RU = RL + IYB - 1;
     static constexpr int right_pitch() {
         int n = KBX + VK;
         while (n % VK != 0 || (P == 32 ? (n / EV) % 2 != 1 : (n / EV) % 4 != 2)) n += EV;
@@ -125,11 +144,12 @@ struct MfmaCfg {
     static constexpr int QP = WZ < 4 ? WZ : 4; // quads per pass (= wavefronts that add and write in a pass)
     static constexpr int RED_ELEMS = QP * WZ * 64 * 4;
     static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
-    static_assert(P % JV == 0 && P % IU == 0, "whole matrices per result tile");
+    static_assert(P % (JV * JYO) == 0 && P % IU == 0, "whole matrices per result tile");
+    static_assert(JYO == 1 || (JV == 1 && NIY == 1), "copies of the x shifts: one left matrix per result tile, one tile along y");
     static_assert(EV % NC == 0, "the instructions of a step are dealt evenly to the accumulator sets");
     static_assert(WZ > 1 && (KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
-    static_assert(PV % VK == 0 && VBAND % VK == 0 && UBAND % VK == 0, "128-bit LDS pieces");
-    static_assert(LX * LY * LV * LU == 64, "lane bookkeeping");
+    static_assert((PV % VK == 0 || JYO > 1) && VBAND % VK == 0 && UBAND % VK == 0, "128-bit LDS pieces");
+    static_assert(LX * LY * LV * LU * WY == 64, "lane bookkeeping");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
@@ -148,10 +168,11 @@ struct BandStager {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
     static constexpr int VK = C::VK, PP = COLS / VK, TOTP = NB * ROWS * PP;
+    static constexpr bool WIDE = PITCH % VK == 0; // rows on 128-bit boundaries of the LDS image: one store per piece, else two of 64 bits
     static constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
     static constexpr int BATCH = ITER < C::SB ? ITER : C::SB;
     static constexpr unsigned NONE = ~0u;
-    static_assert(COLS % VK == 0 && PITCH % VK == 0 && BAND % VK == 0, "128-bit LDS pieces");
+    static_assert(COLS % VK == 0 && COLS <= PITCH && BAND % VK == 0 && (PITCH * sizeof(T)) % 8 == 0, "128-bit pieces, 64-bit LDS stores at least");
     static_assert(ROWS < 4096 && COLS <= 4096 && NB < 255, "packed piece coordinates");
     unsigned gbyte[ITER]; // byte offset of the piece from the stage origin (the element at band 0, row 0, column 0)
     unsigned where[ITER]; // band << 24 | row << 12 | column; NONE: this thread has no piece in this round
@@ -209,7 +230,23 @@ struct BandStager {
 #pragma unroll
             for (int j = 0; j < BATCH; ++j) {
                 const int i = i0 + j;
-                if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) *reinterpret_cast<vec *>(lds + lds_at[i]) = val[j];
+                if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) {
+                    if constexpr (WIDE) {
+                        *reinterpret_cast<vec *>(lds + lds_at[i]) = val[j];
+                    } else {
+                        if constexpr (VK == 2) {
+                            lds[lds_at[i]] = val[j][0];
+                            lds[lds_at[i] + 1] = val[j][1];
+                        } else {
+                            typedef T half_t __attribute__((ext_vector_type(VK / 2)));
+                            half_t lo, hi;
+#pragma unroll
+                            for (int e = 0; e < VK / 2; ++e) lo[e] = val[j][e], hi[e] = val[j][VK / 2 + e];
+                            *reinterpret_cast<half_t *>(lds + lds_at[i]) = lo;
+                            *reinterpret_cast<half_t *>(lds + lds_at[i] + VK / 2) = hi;
+                        }
+                    }
+                }
             }
         }
     }
@@ -321,14 +358,14 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
     // ---- lane coordinates inside a result tile ----
     const int lane = tid & 63;
     const int p = lane % P, kk = lane / P;
-    const int vj = p / C::JX, sxl = p % C::JX; // column j = p: left matrix, x shift
+    const int vj = p / C::JX / C::JYO, yo = p / C::JX % C::JYO, sxl = p % C::JX; // column j = p: left matrix, copy, x shift
     const int ui = p / C::IY, syl = p % C::IY; // row i = p: right matrix, y shift
     // With AL the left bands start at the 128-bit boundary of the matrix rows at or below the tile's first column (x0 is a multiple of
     // 8): every staged piece is then aligned in global memory and, where the width is a multiple of VK, wholly inside or
     // outside the matrix; the lanes read `left_shift` columns further in.
     const int left_shift = C::AL ? ((sxb % VK) + VK) % VK : 0;
-    const T *Vs_lane = Vs + vj * C::VBAND + sxl + C::EV * kk + left_shift;
-    const T *Us_lane = Us + ui * C::UBAND + (C::TYB - 1 - syl) * C::PU + C::EV * kk;
+    const T *Vs_lane = Vs + vj * C::VBAND + yo * C::IY * C::PV + sxl + C::EV * kk + left_shift;
+    const T *Us_lane = Us + ui * C::UBAND + (C::IYB - 1 - syl) * C::PU + C::EV * kk;
 
     acc_t acc[C::TJ][C::TI][C::NC];
 #pragma unroll
@@ -347,32 +384,40 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
     // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner). (Fetching the next stage into
     // registers before the current one is swept, to hide the load latency behind the matrix instructions, measured
     // 2 % slower on large matrices and no faster on small ones: the other blocks of the CU already cover it.)
-    BandStager<C, C::NVB, C::RL, C::PV, C::PV, C::VBAND> left_stager;
+    BandStager<C, C::NVB, C::VROWS, C::PVC, C::PV, C::VBAND> left_stager;
     BandStager<C, C::NUB, C::RU, C::KBX, C::PU, C::UBAND> right_stager; // (the padding columns of a right row are never read)
     left_stager.init(tid, W, HW);
     right_stager.init(tid, W, HW);
     const T *left_first = g.V + (size_t)v_first * HW, *right_first = g.U + (size_t)u_first * HW;
-    for (int yl0 = clo; yl0 < chi; yl0 += C::RL) {
+    // yl0: the left row of the first copy (the base row yb of the header); the last copy is (JYO - 1) * IY rows ahead of it.
+    // Base rows below syb or from syb + IYB + H - 1 on meet no right row.
+    int yl_begin = clo - (C::JYO - 1) * C::IY, yl_end = chi;
+    if (C::JYO > 1) {
+        if (yl_begin < syb) yl_begin = syb;
+        if (yl_end > syb + C::IYB + H - 1) yl_end = syb + C::IYB + H - 1;
+    }
+    for (int yl0 = yl_begin; yl0 < yl_end; yl0 += C::RL) {
         for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
             __syncthreads(); // everyone is done reading the previous stage
             {
-                // left band: rows [yl0, yl0+RL), columns xl = x0 + sxb - shift + col (the 128-bit boundary at or below x0 + sxb)
+                // left band: rows [yl0, yl0+VROWS) of the chunk's rows [clo, chi), columns xl = x0 + sxb - shift + col (the 128-bit boundary at or below x0 + sxb)
                 const int xbase = x0 + sxb - left_shift;
-                // right band: rows yr = yl0 - syb - TYB + 1 + row, columns xr = x0 + col
-                const int yr0 = yl0 - syb - C::TYB + 1;
+                // right band: rows yr = yl0 - syb - IYB + 1 + row, columns xr = x0 + col
+                const int yr0 = yl0 - syb - C::IYB + 1;
                 const int ur_lo = yr0 < 0 ? -yr0 : 0;
                 const int ur_hi = H - yr0 < C::RU ? H - yr0 : C::RU;
-                const int rows_ok = chi - yl0 < C::RL ? chi - yl0 : C::RL;
+                const int vr_lo = clo - yl0 > 0 ? clo - yl0 : 0;
+                const int vr_hi = chi - yl0 < C::VROWS ? chi - yl0 : C::VROWS;
                 const int vc_lo = xbase < 0 ? -xbase : 0;
-                const int vc_hi = W - xbase < C::PV ? W - xbase : C::PV;
+                const int vc_hi = W - xbase < C::PVC ? W - xbase : C::PVC;
                 const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
-                left_stager.stage(Vs, left_first + (ptrdiff_t)yl0 * W + xbase, nbv, 0, rows_ok, vc_lo, vc_hi);
+                left_stager.stage(Vs, left_first + (ptrdiff_t)yl0 * W + xbase, nbv, vr_lo, vr_hi, vc_lo, vc_hi);
                 right_stager.stage(Us, right_first + (ptrdiff_t)yr0 * W + x0, nbu, ur_lo, ur_hi, 0, uc_hi);
             }
             __syncthreads();
-            // left rows of this stage that can overlap the tile's y shifts: yl in [syb, syb + TYB - 1 + H - 1], yl < chi
+            // base rows of this stage whose window of right rows meets the right matrix: yb in [syb, syb + IYB - 1 + H - 1], yb < chi
             int first = syb - yl0;
-            int last = syb + C::TYB + H - 2 - yl0;
+            int last = syb + C::IYB + H - 2 - yl0;
             if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
             if (last > C::RL - 1) last = C::RL - 1;
             const int row0 = first > 0 ? first : 0;
@@ -448,7 +493,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
             for (int e = 0; e < 4; ++e) {
                 const int i = C::Op::row(r0 + e, kk); // result row: right matrix, y shift
                 const int u = u_first + (t / C::NIY) * C::IU + i / C::IY;
-                const int oy = syb + (t % C::NIY) * C::IY + i % C::IY + (H - 1);
+                const int oy = syb + yo * C::IYB + (t % C::NIY) * C::IY + i % C::IY + (H - 1);
                 if (u < u_limit && oy >= 0 && oy < Sy) {
                     const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
                     T *o = g.out + mat_index * out_area + (size_t)oy * Sx + ox;

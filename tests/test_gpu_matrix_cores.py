@@ -103,6 +103,47 @@ def test_all_pairs(oracle, dtype):
     assert any("_l" in k for k in seen), seen  # tiles with left matrices over the columns of a result tile were used
 
 
+def test_tiles_with_copies_of_the_x_shifts(oracle):
+    """The fp32 tiles whose result columns hold 16 x shifts twice, 8 left rows apart (16 x 16 shifts of 4 right matrices): forced by
+    index on shapes around their 8-row offset, the 32-row stages and the 64-bit-aligned rows of their left band, whole and in chunks
+    of left rows that start and end anywhere; the launcher's own choice on a launch they are best for."""
+    xc = load_package()
+    rng = np.random.default_rng(905)
+    indices = []
+    probe = ints(rng, (1, 4, 4), np.float32)
+    for index in range(1, 64):
+        try:
+            xc.run("multimat_right_grouped", probe, probe, 1, n_left=1, n_right=1, params=xc.make_params(specialisation=index))
+        except xc.XcorrError as e:
+            if "does not exist" in e.message:
+                break
+            continue
+        if "_m16x16_" in xc.last_launch()["kernel"]:
+            indices.append(index)
+    assert len(indices) == 2, indices
+    for index in indices:
+        for shape in [(1, 1), (5, 3), (7, 9), (8, 8), (9, 16), (16, 16), (19, 23), (31, 33), (33, 17), (40, 40), (64, 64), (70, 130), (150, 41)]:
+            for n_right in (1, 3, 4, 9):
+                left, right = ints(rng, (1,) + shape, np.float32), ints(rng, (n_right,) + shape, np.float32)
+                exp = oracle.one_to_many(left, right, threads=4)
+                for kw in [{}, dict(rows_per_thread=3), dict(rows_per_thread=8), dict(rows_per_thread=24), dict(rows_per_thread=40, column_chunks=2)]:
+                    say("copies", index, shape, n_right, kw)
+                    got = xc.run("multimat_right_grouped", left, right, n_right, n_left=1, n_right=n_right, params=xc.make_params(specialisation=index, **kw))
+                    rec = xc.last_launch()
+                    bad = np.argwhere(got != exp)
+                    assert bad.size == 0, (index, shape, n_right, kw, rec["kernel"], bad[:3].tolist())
+        left, right = ints(rng, (3, 40, 70), np.float32), ints(rng, (15, 40, 70), np.float32)
+        exp = np.concatenate([oracle.one_to_many(left[l:l + 1], right[l * 5:(l + 1) * 5]) for l in range(3)])
+        assert np.array_equal(xc.run("multimat_right_grouped", left, right, 15, n_left=3, n_right=5, params=xc.make_params(specialisation=index)), exp)
+        exp = oracle.n_to_m(left, right, threads=4)
+        assert np.array_equal(xc.run("multimat_both_grouped", left, right, 45, n_left=3, n_right=15, params=xc.make_params(specialisation=index, rows_per_thread=16)), exp)
+    left, right = rng.standard_normal((1, 128, 128)).astype(np.float32), rng.standard_normal((64, 128, 128)).astype(np.float32)
+    got = xc.run("multimat_right_grouped", left, right, 64, n_left=1, n_right=64)
+    assert "_m16x16_r4" in xc.last_launch()["kernel"], xc.last_launch()["kernel"]
+    sample = [0, 17, 63]
+    assert rel_frob(got[sample], oracle.one_to_many(left, right[sample], threads=4)) <= 1e-5
+
+
 def test_never_and_only(oracle):
     """matrix_cores = 2 keeps the register tiles; both settings give the same integers."""
     xc = load_package()
