@@ -34,7 +34,7 @@ MEASURED_TRAFFIC = {
     ("C4", "multimat_right_grouped/f32_m32x8_r4"): (0.0106e9 + 0.0494e9, "profiles/engine_other_workloads.md"),
     ("C3", "multimat_right_grouped/f32_a8b4_lr8"): (0.0253e9 + 0.1430e9, "profiles/engine_other_workloads.md"),
     ("C4", "multimat_right_grouped/f32_a8b4_lr8"): (0.0114e9 + 0.0619e9, "profiles/engine_other_workloads.md"),
-    ("C5", "multimat_both_grouped/f64_m8x8_l4r4"): (0.0064e9 + 0.1068e9, "profiles/engine_other_workloads.md"),
+    ("C5", "multimat_both_grouped/f64_m8x8_l4r4"): (0.0057e9 + 0.1067e9, "profiles/engine_other_workloads.md"),
     ("C5", "multimat_both_grouped/f64_a8b4_ll4lr8"): (0.0070e9 + 0.1100e9, "profiles/engine_other_workloads.md"),
 }
 

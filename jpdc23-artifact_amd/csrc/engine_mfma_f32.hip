@@ -6,7 +6,9 @@
 
 namespace xcorr {
 
-//                              T   JV IU MJX MJV NIY NIU  RL KBX MINB AL
+//                              T   JV IU MJX MJV NIY NIU  RL KBX MINB AL NC WZ SB JYO
+// (pieces per staging batch SB: four instead of eight frees the registers that spill in some of these and changes no run time by more than
+// 0.4 %, except for the pair tiles below)
 // one pair per block
 using M_32x32 = MfmaCfg<float, 1, 1, 1, 1, 1, 1, 32, 64, 4>;
 using M_64x32 = MfmaCfg<float, 1, 1, 2, 1, 1, 1, 32, 64, 4>;
@@ -19,7 +21,8 @@ using M_16x16_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 32, 32, 3, 0, 1, 4, 8, 2>;
 // (four copies 4 rows apart with 8 right matrices - 8 x 16 shifts, MfmaCfg<float, 1, 8, 1, 1, 1, 1, 32, 32, 3, 0, 1, 4, 8, 4> - measured
 // 2-8 % behind M_16x16_r4 wherever it ran, its eight right bands leave three blocks per CU: not compiled)
 // ... and rows over right, columns over left matrices (n_to_m)
-using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 32, 32, 3, 1>;
+// (stages of 16 rows and four pieces per staging batch: 112 registers, four blocks per CU; 32 rows at three blocks 4-10 % slower)
+using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 16, 32, 4, 1, 1, 4, 4>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)
@@ -27,7 +30,7 @@ static const EngineSpec specs[] = {
     make_spec<M_64x32>("f32_m64x32", 0.82, 1.0),
     make_spec<M_32x8_r4>("f32_m32x8_r4", 0.82, 1.0),
     make_spec<M_32x8_r8>("f32_m32x8_r8", 0.88, 1.0),
-    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.96, 1.0),
+    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.90, 1.0),
     make_spec<M_16x16_r4>("f32_m16x16_r4", 0.855, 1.0),
     make_spec<M_16x16_r8>("f32_m16x16_r8", 0.92, 1.0),
 };
