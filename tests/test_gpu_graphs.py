@@ -1,5 +1,5 @@
 """HIP graph capture of the C ABI's launches: a captured sequence (clear kernel, split-row family with atomics, the
-grouped family with its own clear and row split, the overlap-wise kernel) is replayed several times with eager work and
+grouped family with its own clear and row split on register and on matrix-core tiles, the overlap-wise kernel) is replayed several times with eager work and
 synchronisations between the replays and with fresh inputs each time; every replay must equal the oracle exactly."""
 import ctypes
 
@@ -25,7 +25,7 @@ def test_captured_sequence_replays_with_fresh_inputs(oracle, dtype):
     item = np.dtype(dtype).itemsize
     d_left, d_right = xc.DeviceBuffer(48 * 40 * item), xc.DeviceBuffer(48 * 40 * item)
     d_many = xc.DeviceBuffer(6 * 48 * 40 * item)
-    outs = {k: xc.DeviceBuffer(n * out_elems * item) for k, n in [("split_row", 1), ("grouped", 1), ("overlap_wise", 1), ("many", 6)]}
+    outs = {k: xc.DeviceBuffer(n * out_elems * item) for k, n in [("split_row", 1), ("grouped", 1), ("overlap_wise", 1), ("many", 6), ("cores", 1), ("many_cores", 6)]}
 
     def upload(buf, a):
         a = np.ascontiguousarray(a)
@@ -36,15 +36,21 @@ def test_captured_sequence_replays_with_fresh_inputs(oracle, dtype):
         xc.launch("split_row", d_left, d_right, outs["split_row"], 40, 48, 1, 1, dtype, xc.make_params(rows_per_thread=7), stream)
         xc.launch("grouped_overlap", d_left, d_right, outs["grouped"], 40, 48, 1, 1, dtype, None, stream)
         xc.launch("overlap_wise", d_left, d_right, outs["overlap_wise"], 40, 48, 1, 1, dtype, None, stream)
-        xc.launch("multimat_right_grouped", d_left, d_many, outs["many"], 40, 48, 1, 6, dtype, xc.make_params(rows_per_thread=18), stream)
+        xc.launch("grouped_overlap", d_left, d_right, outs["cores"], 40, 48, 1, 1, dtype, xc.make_params(matrix_cores=1, rows_per_thread=16), stream)
+        assert xc.last_launch()["matrix_cores"] == 1 and xc.last_launch()["uses_atomics"] == 1
+        xc.launch("multimat_right_grouped", d_left, d_many, outs["many_cores"], 40, 48, 1, 6, dtype, xc.make_params(matrix_cores=1), stream)
+        assert xc.last_launch()["matrix_cores"] == 1
+        xc.launch("multimat_right_grouped", d_left, d_many, outs["many"], 40, 48, 1, 6, dtype, xc.make_params(matrix_cores=2, rows_per_thread=18), stream)
 
     def check(left, right, many, what):
         exp = oracle.one_to_one(left, right)[0]
-        for k in ("split_row", "grouped", "overlap_wise"):
+        for k in ("split_row", "grouped", "overlap_wise", "cores"):
             got = outs[k].to_numpy((95, 79), dtype)
             np.testing.assert_array_equal(got, exp, err_msg=f"{what} {k}")
         got = outs["many"].to_numpy((6, 95, 79), dtype)
         np.testing.assert_array_equal(got, oracle.one_to_many(left, many), err_msg=f"{what} many")
+        got = outs["many_cores"].to_numpy((6, 95, 79), dtype)
+        np.testing.assert_array_equal(got, oracle.one_to_many(left, many), err_msg=f"{what} many, matrix cores")
 
     left, right, many = ints(rng, shape, dtype), ints(rng, shape, dtype), ints(rng, (6,) + shape, dtype)
     upload(d_left, left), upload(d_right, right), upload(d_many, many)
