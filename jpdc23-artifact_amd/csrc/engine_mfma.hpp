@@ -24,7 +24,8 @@
 // stage's steps to the wavefronts (mfma_stage) are this file's.
 //
 // Result layout of the instructions (lane l, accumulator element r): column j = l % P; row i = 8 * (r / 4) + 4 * (l / 32) + r % 4
-// for the fp32 instruction and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs.
+// for the fp32 instruction and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs (two
+// runs of 64 bytes in different result rows for the tiles whose columns hold the x shifts twice, see JYO_ below).
 #pragma once
 
 #include "engine.hpp"
