@@ -25,6 +25,10 @@ using M_16x16_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 16, 32, 4, 0, 1, 4, 4, 2>;
 // ... and rows over right, columns over left matrices (n_to_m)
 // (stages of 16 rows and four pieces per staging batch: 112 registers, four blocks per CU; 32 rows at three blocks 4-10 % slower)
 using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 16, 32, 4, 1, 1, 4, 4>;
+// two result tiles per wavefront over eight right matrices: half the work items, each staging 1.5 x the bands for twice the products (128
+// registers, four blocks per CU): 6-16 % faster than the 4 x 4 tile on 16x16 ... 64x64 matrices, level at 128x128. (Eight left matrices instead:
+// 2-4 % behind this one; the fp64 counterparts need 168 registers or 64 KB of LDS and are 8-14 % slower than the fp64 4 x 4 tile: not compiled.)
+using M_8x8_l4r8 = MfmaCfg<float, 4, 4, 1, 1, 1, 2, 16, 32, 4, 1, 1, 4, 4>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)
@@ -35,6 +39,7 @@ static const EngineSpec specs[] = {
     make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.90, 1.0),
     make_spec<M_16x16_r4>("f32_m16x16_r4", 0.855, 1.0),
     make_spec<M_16x16_r8>("f32_m16x16_r8", 0.875, 1.0),
+    make_spec<M_8x8_l4r8>("f32_m8x8_l4r8", 0.89, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f32(int *count) {
