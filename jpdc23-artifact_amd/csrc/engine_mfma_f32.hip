@@ -37,8 +37,8 @@ static const EngineSpec specs[] = {
     make_spec<M_32x8_r4>("f32_m32x8_r4", 0.82, 1.0),
     make_spec<M_32x8_r8>("f32_m32x8_r8", 0.84, 1.0),
     make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.90, 1.0),
-    make_spec<M_16x16_r4>("f32_m16x16_r4", 0.855, 1.0),
-    make_spec<M_16x16_r8>("f32_m16x16_r8", 0.875, 1.0),
+    make_spec<M_16x16_r4>("f32_m16x16_r4", 0.83, 1.0),
+    make_spec<M_16x16_r8>("f32_m16x16_r8", 0.85, 1.0),
     make_spec<M_8x8_l4r8>("f32_m8x8_l4r8", 0.89, 1.0),
 };
 

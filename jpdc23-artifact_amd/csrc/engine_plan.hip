@@ -157,8 +157,9 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     // lanes over matrices; it has no window of A right rows to fill before a chunk's first row)
     const bool f32 = s.elem_bytes == 4, lanes_over_matrices = s.MFMA ? s.NVB() * s.NUB() > 1 : s.LV * s.LU > 1;
     const int window = s.MFMA ? 0 : s.A - 1;
-    // A matrix-core tile whose columns hold copies of the x shifts some rows apart (TYB > TYW) sweeps the rows of its first copy only,
-    // from `copies` rows before a chunk's first row on: about copies / 2 fewer than its shifts overlap when whole.
+    // A matrix-core tile whose columns hold copies of the x shifts some rows apart (TYB > TYW) sweeps the left rows of its first copy,
+    // from `copies` rows before a chunk's first row on: as many as its shifts overlap when whole (up to `copies` more for the tiles
+    // around y shift 0), `copies` more than the chunk when cut.
     const int copies = s.MFMA ? s.TYB() - s.TYW() : 0;
     const double t_block = 4.41, tau = 1.07, e_full = 0.954, t_stage = 0.209, k_tail = 0.281;
     const double t_clear = f32 ? 1.49 : 0.0, t_atomic = f32 ? 0.0462 : 0.0811;
@@ -173,7 +174,7 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     const double live = plan.x_chunks > 1 ? std::fmin(plan.x_chunks, std::ceil(cols_tile / plan.x_chunk_cols)) : 1.0;
     const double cols_avg = cols_tile / live, cols_max = plan.x_chunks > 1 ? std::fmin(W, plan.x_chunk_cols) : W;
     const double rows_tile = std::fmin(H, H * (H + TYW) / (plan.nty * TYW));
-    const double rows_avg = (split && rc < rows_tile ? rc + copies : rows_tile - 0.5 * copies) + window;
+    const double rows_avg = (split && rc < rows_tile ? rc + copies : rows_tile) + window;
     const double rows_max = (split && rc < H ? rc + copies : H + 0.5 * copies) + window;
     const double per_element = (double)s.NV * s.NU * s.A * s.B / s.WZ * s.issue_factor;
     const double inst_avg = per_element * rows_avg * cols_avg, inst_max = per_element * rows_max * cols_max;
@@ -224,6 +225,9 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         }
         if (rq.spec_index == 0) {
             if (rq.matrix_cores == 1 ? !s.MFMA : rq.matrix_cores == 2 ? s.MFMA != 0 : false) continue;
+            // The tiles whose columns hold copies of the x shifts win up to about 256x256 matrices (2-7 % over their 32 x 8
+            // counterparts) and measured level at 300x300, 3-14 % behind at 384x384 ... 1024x1024, which the model does not show.
+            if (s.MFMA && s.TYB() != s.TYW() && (double)rq.W * rq.H > 300.0 * 300.0) continue;
             if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
             if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
             if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
