@@ -50,6 +50,10 @@ struct EngineArgs {
     int total_items;    // nvg * nug * nworkers_y * ntx * x_chunks
     int x_chunks;       // >1: the right columns a tile overlaps are cut into chunks of x_chunk_cols (atomic adds)
     int x_chunk_cols;   // multiple of K * WZ
+    // Work queue of a persistent launch (matrix-core sweep): queue[0] counts the work items handed out beyond the first one of
+    // every block, queue[1] the blocks that are done; both are zero before the launch and the last block to finish zeroes
+    // them again. nullptr: block b takes the items b, b + gridDim.x, ... (with one block per work item: exactly one).
+    unsigned *queue;
 };
 
 // WZ_ > 1: the WZ_ wavefronts of a workgroup (WX_ = WY_ = 1) work on the SAME tile of shifts and
@@ -166,13 +170,12 @@ struct WorkItem {
     int xr_lo, xr_hi, w_hi;        // right columns [xr_lo, xr_hi) to reduce over; w_hi bounds what a partial last stage may sweep
 };
 
-// Decodes blockIdx.x into a work item; false when the block has nothing to do (surplus workers of the rectangle
+// Decodes work item number `item` (in launch order); false when there is nothing to do for it (surplus workers of the rectangle
 // distribution, column chunks beyond a narrow tile's overlap). C supplies the block tile (TXB, TYB), the matrices per
 // block (NVB, NUL, NUB) and the column granule K.
 template <class C, typename T>
-__device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, WorkItem &wi) {
+__device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, int item, WorkItem &wi) {
     const int W = g.W, H = g.H;
-    int item = (int)blockIdx.x;
     if (item >= g.total_items) return false;
     const int xch = item % g.x_chunks;
     item /= g.x_chunks;
@@ -475,7 +478,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void engine_kernel(EngineArgs<typen
 
     // ---- the work item (uniform over the threads that share it) ----
     WorkItem wi;
-    if (!decode_work_item<C>(g, wi)) return;
+    if (!decode_work_item<C>(g, (int)blockIdx.x, wi)) return;
     const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
     const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
 

@@ -28,6 +28,8 @@
 // runs of 64 bytes in different result rows for the tiles whose columns hold the x shifts twice, see JYO_ below).
 #pragma once
 
+#include <type_traits>
+
 #include "engine.hpp"
 
 namespace xcorr {
@@ -66,14 +68,11 @@ constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 
 // P / JYO_ x shifts by IY * JYO_ y shifts of one left matrix instead of P by IY (a squarer tile sweeps fewer rows and columns that
 // only some of its shifts overlap). The copies come from the same LDS band, IY rows further down: they cost (JYO_ - 1) * IY
 // more rows per band and per chunk of left rows, no staging.
-// AL_ = 1: the left bands start on a 128-bit boundary of the matrix rows (see mfma_kernel); costs up to VK - 1 more columns per
-// left row, saves the element-wise assembly of pieces at the matrix edges: for tiles that mostly run on small matrices.
-template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int AL_ = 0, int NC_ = 1, int WZ_ = 4,
-          int SB_ = 8, int JYO_ = 1>
+template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int NC_ = 1, int WZ_ = 4, int JYO_ = 1>
 struct MfmaCfg {
     using value_type = T;
     using Op = MfmaOp<T>;
-    static constexpr int MFMA = 1, PG = 0, DB = 0, SB = SB_;
+    static constexpr int MFMA = 1, PG = 0, DB = 0;
     static constexpr int P = Op::P, ACC = Op::ACC, KS = 64 / P;
     static constexpr int VK = 16 / (int)sizeof(T);
     static constexpr int EV = Op::EV;   // consecutive elements a lane reads per operand and step = instructions per step and result tile
@@ -86,7 +85,7 @@ struct MfmaCfg {
     static constexpr int NVB = JV * MJV, NUL = IU * NIU, NUB = NUL;
     // (the copies of the x shifts are reported as half or quarter wavefronts along y)
     static constexpr int WX = 1, WY = JYO, WZ = WZ_, NWAVES = WZ, NT = 64 * NWAVES;
-    static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_, AL = AL_;
+    static constexpr int RL = RL_, KBX = KBX_, MINB = MINB_, NC = NC_;
     // what the launch record and the planner call the tile: shifts and matrices per lane, lanes over each
     static constexpr int A = (1 << popcount_c(Op::REG_BITS & (IY - 1))) * NIY;
     static constexpr int B = MJX;
@@ -102,7 +101,7 @@ struct MfmaCfg {
     // with IY rows a multiple of that apart: 0.35 conflict cycles per LDS cycle). No multiple of 128 bits does that for 8 rows:
     // such a band keeps its rows on 64-bit boundaries only and is filled with 64-bit LDS stores.
     static constexpr int BANK_ELEMS = 256 / (int)sizeof(T);
-    static constexpr int PVC = (TXB + KBX - 1 + (AL ? VK - 1 : 0) + VK - 1) / VK * VK; // columns of a left band
+    static constexpr int PVC = (TXB + KBX - 1 + (VK - 1) + VK - 1) / VK * VK; // columns of a left band
     static constexpr int left_pitch() {
         int n = PVC;
         if (JYO > 1)
@@ -144,7 +143,8 @@ struct MfmaCfg {
     static constexpr int NQ = TJ * TI * ACC / 4;
     static constexpr int QP = WZ < 4 ? WZ : 4; // quads per pass (= wavefronts that add and write in a pass)
     static constexpr int RED_ELEMS = QP * WZ * 64 * 4;
-    static constexpr int LDS_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
+    static constexpr int BAND_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
+    static constexpr int LDS_BYTES = BAND_BYTES + 16; // + two slots through which thread 0 hands the block its next work item
     static_assert(P % (JV * JYO) == 0 && P % IU == 0, "whole matrices per result tile");
     static_assert(JYO == 1 || (JV == 1 && NIY == 1), "copies of the x shifts: one left matrix per result tile, one tile along y");
     static_assert(EV % NC == 0, "the instructions of a step are dealt evenly to the accumulator sets");
@@ -154,102 +154,192 @@ struct MfmaCfg {
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
 };
 
-// Staging of NB bands (ROWS rows x COLS columns each; row pitch PITCH and band stride BAND in LDS; matrices `mat_stride`
-// apart in global memory) with everything that does not change from stage to stage worked out once per block: thread
-// `tid` moves the 128-bit pieces p = tid + i * NT, piece p being (band, row, column piece) = (p / (PP * ROWS),
-// (p / PP) % ROWS, p % PP), and keeps per piece its byte offset from the stage's origin in global memory, its LDS offset
-// and its coordinates. A stage that lies wholly inside the matrices (the rule away from the matrix edges) is then one
-// load with a scalar base and one LDS store per piece, no address arithmetic; the other stages zero what lies outside
-// [row_lo, row_hi) x [col_lo, col_hi) or belongs to a band that does not exist and assemble pieces that straddle a column
-// bound element by element. (Every instruction a wavefront issues next to the matrix instructions of the other
-// wavefronts of its SIMD costs the matrix pipeline about two cycles; the generic staging of the register-tile sweep
-// issued as many vector and scalar instructions per stage as the sweep issues matrix instructions.)
-template <class C, int NB, int ROWS, int COLS, int PITCH, int BAND>
-struct BandStager {
+// Staging of NB bands (ROWS rows x COLS columns each; row pitch PITCH and band stride BAND in LDS) by loads that write LDS
+// directly (buffer_load ... lds: no registers, no LDS store instructions, completion counted by vmcnt). One such instruction
+// moves GRAN bytes per lane to 64 consecutive pieces of LDS, so the image of a band is taken as a run of pieces
+// q = 0 .. ROWS * PITCH / PE - 1 (PE elements each), piece q being (row, column) = (q / PP, (q % PP) * PE); lane l of copy j
+// fetches piece 64 j + l. Every band has a buffer descriptor of its own that covers exactly the rows that may be read (the
+// matrix, or the chunk of left rows of the work item): a piece of a row outside them has an offset below zero or beyond the
+// descriptor's size and the hardware writes zeros for it - the zero padding above and below the matrices costs nothing. Left and
+// right of the matrices the offset would fall into a neighbouring row: there (and only in stages that reach over the edge) the
+// lane's column is compared and the offset replaced by one that is out of range. A piece that straddles the right edge (widths
+// that are not a multiple of the piece) is loaded whole and its tail zeroed afterwards (fix_right_edge).
+// Per lane and copy two registers are kept: byte offset and column of the piece relative to the stage origin. A wavefront copies
+// the bands w, w + WZ, ... whole (NB a multiple of WZ), or the copies w, w + WZ, ... of the only band.
+// GRAN = 4 (one fp32 element per lane) serves images whose rows are not 128 bits apart.
+using buffer_rsrc = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ buffer_rsrc make_rsrc(const void *base, unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), (short)0, (int)bytes, 0x00020000);
+}
+template <int GRAN>
+__device__ __forceinline__ void dma_piece(buffer_rsrc r, void *lds_wave_base, unsigned voffset) {
+    // (the size must be a literal for the builtin)
+    if constexpr (GRAN == 16)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_wave_base, 16, (int)voffset, 0, 0, 0);
+    else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (__attribute__((address_space(3))) void *)lds_wave_base, 4, (int)voffset, 0, 0, 0);
+    static_assert(GRAN == 16 || GRAN == 4, "piece sizes the instruction has");
+}
+
+template <class C, int NB, int ROWS, int COLS, int PITCH, int BAND, int GRAN>
+struct BandDma {
+    using T = typename C::value_type;
+    static constexpr int EB = (int)sizeof(T);
+    static constexpr int PE = GRAN / EB;        // elements per piece
+    static constexpr int PP = PITCH / PE;       // pieces per image row
+    static constexpr int Q = ROWS * PP;         // pieces of a band image (the spare row behind them is not loaded)
+    static constexpr int J = (Q + 63) / 64;     // wavefront-wide copies per band
+    static constexpr bool OWN = NB >= C::WZ;    // a wavefront copies whole bands
+    static constexpr int NBW = OWN ? NB / C::WZ : 1;
+    static constexpr int TJ = OWN ? J : (J + C::WZ - 1) / C::WZ;
+    static constexpr unsigned OUTSIDE = 0x80000000u; // an offset no descriptor covers (a matrix has at most 2^31 bytes)
+    static_assert(GRAN % EB == 0 && PITCH % PE == 0 && (BAND * EB) % GRAN == 0, "whole pieces");
+    static_assert(NB == 1 || NB % C::WZ == 0, "bands per block: one, or a multiple of the wavefronts");
+    static_assert(COLS <= PITCH, "image rows hold the columns");
+    unsigned lane_off[TJ]; // (row * W + column) * EB of the lane's piece in copy t
+    int lane_col[TJ];      // its first column; beyond the image's columns (padding of the pitch): a number no matrix is wide
+    buffer_rsrc rsrc[NBW];
+
+    // copy t of this wavefront is copy j of its band(s)
+    __device__ __forceinline__ static int copy_index(int t, int wave) { return OWN ? t : wave + t * C::WZ; }
+
+    __device__ __forceinline__ void init(int lane, int wave, int W) {
+#pragma unroll
+        for (int t = 0; t < TJ; ++t) {
+            const int q = 64 * copy_index(t, wave) + lane;
+            const int row = q / PP, col = (q % PP) * PE;
+            lane_off[t] = (unsigned)((row * W + col) * EB);
+            lane_col[t] = col < COLS ? col : (1 << 28);
+        }
+    }
+    // The bands of a work item: band b is the matrix `first + b * mat_stride`, of which the rows [row_lo, row_lo + rows) exist
+    // (the others read as zero); bands from `nbands` on do not exist.
+    __device__ __forceinline__ void set_item(const T *first, size_t mat_stride, int W, int row_lo, int rows, int nbands, int wave) {
+#pragma unroll
+        for (int i = 0; i < NBW; ++i) {
+            const int b = OWN ? wave + i * C::WZ : 0;
+            rsrc[i] = make_rsrc(first + (size_t)b * mat_stride + (size_t)row_lo * W, b < nbands ? (unsigned)rows * (unsigned)W * EB : 0u);
+        }
+    }
+    // Stage whose image row 0, column 0 is row `row0` (relative to row_lo of set_item), column `col0` of the matrices.
+    template <bool CHECK>
+    __device__ __forceinline__ void copy(T *lds, int W, int row0, int col0, int lane, int wave) const {
+        const unsigned origin = (unsigned)((row0 * W + col0) * EB);
+#pragma unroll
+        for (int i = 0; i < NBW; ++i) {
+            T *band = lds + (OWN ? wave + i * C::WZ : 0) * BAND;
+#pragma unroll
+            for (int t = 0; t < TJ; ++t) {
+                const int j = copy_index(t, wave);
+                if (!OWN && t == TJ - 1 && j >= J) continue; // (wavefront-uniform)
+                unsigned voffset = lane_off[t] + origin;
+                if (CHECK) voffset = (unsigned)(col0 + lane_col[t]) < (unsigned)W ? voffset : OUTSIDE;
+                char *dst = reinterpret_cast<char *>(band) + j * 64 * GRAN;
+                if (t == TJ - 1 && Q % 64 != 0) {
+                    // the last copy of a band: lanes behind the image's end must not write (the next band starts there)
+                    if (64 * j + lane < Q) dma_piece<GRAN>(rsrc[i], dst, voffset);
+                } else {
+                    dma_piece<GRAN>(rsrc[i], dst, voffset);
+                }
+            }
+        }
+    }
+    __device__ __forceinline__ void stage(T *lds, int W, int row0, int col0, int lane, int wave) const {
+        // (with the padding of the pitch inside the matrix too, no lane needs its column checked)
+        if (col0 >= 0 && col0 + PITCH <= W)
+            copy<false>(lds, W, row0, col0, lane, wave);
+        else
+            copy<true>(lds, W, row0, col0, lane, wave);
+    }
+    // After the copies have landed: a piece that begins inside the matrix and ends beyond its last column has brought the
+    // first elements of the next row along; they become the zeros that belong there. Only for widths that are not a multiple of
+    // the piece, in stages that hold the last column.
+    __device__ __forceinline__ void fix_right_edge(T *lds, int W, int col0, int lane, int wave) const {
+        if (PE == 1 || W % PE == 0 || col0 + COLS <= W) return;
+#pragma unroll
+        for (int i = 0; i < NBW; ++i) {
+            T *band = lds + (OWN ? wave + i * C::WZ : 0) * BAND;
+#pragma unroll
+            for (int t = 0; t < TJ; ++t) {
+                const int j = copy_index(t, wave);
+                const int q = 64 * j + lane, col = col0 + lane_col[t];
+                if (q < Q && j < J && col < W && col + PE > W) {
+#pragma unroll
+                    for (int e = 1; e < PE; ++e)
+                        if (col + e >= W) band[q * PE + e] = T(0);
+                }
+            }
+        }
+    }
+};
+
+// One band (ROWS rows x COLS columns, row pitch PITCH) whose image rows are only 64 bits apart in LDS - the left band of the tiles
+// with copies of the x shifts - goes through registers: 128-bit buffer loads with the same descriptor (rows outside the work
+// item's read as zero), two 64-bit LDS stores per piece. The band starts at any column: in stages that reach over the left or
+// right edge of the matrix a piece may lie partly outside, and its elements are zeroed one by one before they are stored.
+template <class C, int ROWS, int COLS, int PITCH>
+struct BandLoad {
     using T = typename C::value_type;
     using vec = typename vec128<T>::type;
-    static constexpr int VK = C::VK, PP = COLS / VK, TOTP = NB * ROWS * PP;
-    static constexpr bool WIDE = PITCH % VK == 0; // rows on 128-bit boundaries of the LDS image: one store per piece, else two of 64 bits
-    static constexpr int ITER = (TOTP + C::NT - 1) / C::NT;
-    static constexpr int BATCH = ITER < C::SB ? ITER : C::SB;
-    static constexpr unsigned NONE = ~0u;
-    static_assert(COLS % VK == 0 && COLS <= PITCH && BAND % VK == 0 && (PITCH * sizeof(T)) % 8 == 0, "128-bit pieces, 64-bit LDS stores at least");
-    static_assert(ROWS < 4096 && COLS <= 4096 && NB < 255, "packed piece coordinates");
-    unsigned gbyte[ITER]; // byte offset of the piece from the stage origin (the element at band 0, row 0, column 0)
-    unsigned where[ITER]; // band << 24 | row << 12 | column; NONE: this thread has no piece in this round
-    int lds_at[ITER];     // element offset in the LDS image
-    __device__ __forceinline__ void init(int tid, int W, size_t mat_stride) {
+    static constexpr int EB = (int)sizeof(T), VK = C::VK, PPC = COLS / VK, TOT = ROWS * PPC, ITER = (TOT + C::NT - 1) / C::NT;
+    static constexpr unsigned OUTSIDE = 0x80000000u;
+    static_assert(COLS % VK == 0 && (PITCH * EB) % 8 == 0 && VK == 4, "pieces of four elements, rows on 64-bit boundaries");
+    unsigned lane_off[ITER];
+    int lane_col[ITER];
+    int lds_at[ITER]; // element offset in the image
+    buffer_rsrc rsrc;
+    __device__ __forceinline__ void init(int tid, int W) {
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {
             const int p = tid + i * C::NT;
-            const int col = (p % PP) * VK, row = (p / PP) % ROWS, band = p / (PP * ROWS);
-            const bool have = p < TOTP;
-            gbyte[i] = have ? (unsigned)(((size_t)band * mat_stride + (size_t)row * W + col) * sizeof(T)) : 0u;
-            where[i] = have ? ((unsigned)band << 24 | (unsigned)row << 12 | (unsigned)col) : NONE;
-            lds_at[i] = have ? band * BAND + row * PITCH + col : 0;
+            const int row = p / PPC, col = (p % PPC) * VK;
+            lane_off[i] = (unsigned)((row * W + col) * EB);
+            lane_col[i] = col;
+            lds_at[i] = row * PITCH + col;
         }
     }
-    // `origin`: address of (band 0, row 0, column 0) of the stage; it may lie outside the matrix where the bounds exclude
-    // the elements there (it is only offset, never read through, for those)
-    __device__ __forceinline__ void stage(T *lds, const T *origin, int nbands, int row_lo, int row_hi, int col_lo, int col_hi) const {
-        const char *base = reinterpret_cast<const char *>(origin);
-        const bool interior = nbands >= NB && row_lo <= 0 && row_hi >= ROWS && col_lo <= 0 && col_hi >= COLS;
+    __device__ __forceinline__ void set_item(const T *first, int W, int row_lo, int rows, int nbands) {
+        rsrc = make_rsrc(first + (size_t)row_lo * W, nbands > 0 ? (unsigned)rows * (unsigned)W * EB : 0u);
+    }
+    template <bool CHECK>
+    __device__ __forceinline__ void copy(T *lds, int W, int row0, int col0, int tid) const {
+        typedef unsigned uvec __attribute__((ext_vector_type(4)));
+        typedef T half_t __attribute__((ext_vector_type(VK / 2)));
+        const unsigned origin = (unsigned)((row0 * W + col0) * EB);
+        uvec val[ITER];
 #pragma unroll
-        for (int i0 = 0; i0 < ITER; i0 += BATCH) {
-            vec val[BATCH];
-            if (interior) {
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j) {
-                    const int i = i0 + j;
-                    if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) __builtin_memcpy(&val[j], base + gbyte[i], sizeof(vec)); // element-aligned only
-                }
-            } else {
-                // pieces that straddle a column bound exist only where a bound is not a multiple of VK (matrices whose
-                // width is not; the stage origins themselves are kept on 128-bit boundaries)
-                const bool ragged = col_lo % VK != 0 || col_hi % VK != 0;
-#pragma unroll
-                for (int j = 0; j < BATCH; ++j) {
-                    const int i = i0 + j;
-                    vec v;
-#pragma unroll
-                    for (int e = 0; e < VK; ++e) v[e] = T(0);
-                    if (i < ITER) {
-                        const unsigned w = where[i];
-                        const int col = (int)(w & 0xFFFu), row = (int)((w >> 12) & 0xFFFu), band = (int)(w >> 24); // NONE: band 255
-                        const bool in_rows = band < nbands && row >= row_lo && row < row_hi;
-                        const T *q = reinterpret_cast<const T *>(base + gbyte[i]);
-                        if (in_rows && col >= col_lo && col + VK <= col_hi) __builtin_memcpy(&v, q, sizeof(vec));
-                        if (ragged && in_rows && (col < col_lo || col + VK > col_hi) && col + VK > col_lo && col < col_hi) {
-#pragma unroll
-                            for (int e = 0; e < VK; ++e)
-                                if (col + e >= col_lo && col + e < col_hi) v[e] = q[e];
-                        }
-                    }
-                    val[j] = v;
-                }
+        for (int i = 0; i < ITER; ++i) {
+            if ((i + 1) * C::NT > TOT && tid + i * C::NT >= TOT) continue;
+            unsigned voffset = lane_off[i] + origin;
+            if (CHECK) {
+                const int cs = col0 + lane_col[i];
+                voffset = cs > -VK && cs < W ? voffset : OUTSIDE;
             }
-#pragma unroll
-            for (int j = 0; j < BATCH; ++j) {
-                const int i = i0 + j;
-                if (i < ITER && ((i + 1) * C::NT <= TOTP || where[i] != NONE)) {
-                    if constexpr (WIDE) {
-                        *reinterpret_cast<vec *>(lds + lds_at[i]) = val[j];
-                    } else {
-                        if constexpr (VK == 2) {
-                            lds[lds_at[i]] = val[j][0];
-                            lds[lds_at[i] + 1] = val[j][1];
-                        } else {
-                            typedef T half_t __attribute__((ext_vector_type(VK / 2)));
-                            half_t lo, hi;
-#pragma unroll
-                            for (int e = 0; e < VK / 2; ++e) lo[e] = val[j][e], hi[e] = val[j][VK / 2 + e];
-                            *reinterpret_cast<half_t *>(lds + lds_at[i]) = lo;
-                            *reinterpret_cast<half_t *>(lds + lds_at[i] + VK / 2) = hi;
-                        }
-                    }
-                }
-            }
+            val[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voffset, 0, 0);
         }
+#pragma unroll
+        for (int i = 0; i < ITER; ++i) {
+            if ((i + 1) * C::NT > TOT && tid + i * C::NT >= TOT) continue;
+            vec v;
+            __builtin_memcpy(&v, &val[i], sizeof(v));
+            if (CHECK) {
+                const int cs = col0 + lane_col[i];
+#pragma unroll
+                for (int e = 0; e < VK; ++e)
+                    if ((unsigned)(cs + e) >= (unsigned)W) v[e] = T(0);
+            }
+            half_t lo, hi;
+#pragma unroll
+            for (int e = 0; e < VK / 2; ++e) lo[e] = v[e], hi[e] = v[VK / 2 + e];
+            *reinterpret_cast<half_t *>(lds + lds_at[i]) = lo;
+            *reinterpret_cast<half_t *>(lds + lds_at[i] + VK / 2) = hi;
+        }
+    }
+    __device__ __forceinline__ void stage(T *lds, int W, int row0, int col0, int tid) const {
+        if (col0 >= 0 && col0 + COLS <= W)
+            copy<false>(lds, W, row0, col0, tid);
+        else
+            copy<true>(lds, W, row0, col0, tid);
     }
 };
 
@@ -338,6 +428,12 @@ __device__ __forceinline__ void mfma_stage(const typename C::value_type *Vs_lane
     }
 }
 
+// One block = four wavefronts that take work items one after the other. A launch is either one block per work item
+// (gridDim.x = total_items, g.queue == nullptr) or PERSISTENT: as many blocks as the device holds at a time, each taking its own
+// index as first item and every further one from the launch's queue counter (g.queue), i.e. in launch order - heaviest first -
+// as blocks become free, which is what the hardware's own dispatch does with one block per item, minus what a fresh workgroup costs
+// (measured on MI355X: 10 microseconds between the end of a block and the first instruction of its successor in the same slot,
+// plus the set-up below; a work item of the 64x64 matrices lasts 35).
 template <class C>
 __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typename C::value_type> g) {
     using T = typename C::value_type;
@@ -345,165 +441,218 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
     using acc_t = typename C::Op::acc_t;
     constexpr int VK = C::VK, K = C::K, P = C::P;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    // Everything outside the sweep is latency (address arithmetic, loads, barriers) and a few instructions; the sweeps of the
+    // other wavefronts of the SIMD are long runs of matrix instructions that the arbiter would otherwise serve first.
+    __builtin_amdgcn_s_setprio(2);
     const int tid = (int)threadIdx.x;
     const int group = __builtin_amdgcn_readfirstlane(tid >> 6); // which share of the column chunks
     T *Vs = reinterpret_cast<T *>(smem_raw);
     T *Us = Vs + C::NVB * C::VBAND;
+    int *handover = reinterpret_cast<int *>(smem_raw + C::BAND_BYTES); // two slots behind the bands: the next item, alternating
     const int W = g.W, H = g.H;
-
-    WorkItem wi;
-    if (!decode_work_item<C>(g, wi)) return;
-    const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
-    const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
+    const size_t HW = (size_t)W * H;
+    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
+    const size_t out_area = (size_t)Sx * Sy;
 
     // ---- lane coordinates inside a result tile ----
     const int lane = tid & 63;
     const int p = lane % P, kk = lane / P;
     const int vj = p / C::JX / C::JYO, yo = p / C::JX % C::JYO, sxl = p % C::JX; // column j = p: left matrix, copy, x shift
     const int ui = p / C::IY, syl = p % C::IY; // row i = p: right matrix, y shift
-    // With AL the left bands start at the 128-bit boundary of the matrix rows at or below the tile's first column (x0 is a multiple of
-    // 8): every staged piece is then aligned in global memory and, where the width is a multiple of VK, wholly inside or
-    // outside the matrix; the lanes read `left_shift` columns further in.
-    const int left_shift = C::AL ? ((sxb % VK) + VK) % VK : 0;
-    const T *Vs_lane = Vs + vj * C::VBAND + yo * C::IY * C::PV + sxl + C::EV * kk + left_shift;
+    const T *Vs_lane0 = Vs + vj * C::VBAND + yo * C::IY * C::PV + sxl + C::EV * kk;
     const T *Us_lane = Us + ui * C::UBAND + (C::IYB - 1 - syl) * C::PU + C::EV * kk;
 
-    acc_t acc[C::TJ][C::TI][C::NC];
-#pragma unroll
-    for (int s = 0; s < C::TJ; ++s)
-#pragma unroll
-        for (int t = 0; t < C::TI; ++t)
-#pragma unroll
-            for (int c = 0; c < C::NC; ++c)
-#pragma unroll
-                for (int r = 0; r < C::ACC; ++r) acc[s][t][c][r] = T(0);
+    // (the left band of the tiles with copies of the x shifts has rows that are not 128 bits apart: through registers)
+    constexpr bool LEFT_DMA = C::PV % VK == 0;
+    using LeftDma = BandDma<C, C::NVB, C::VROWS, C::PVC, C::PV, C::VBAND, 16>;
+    using LeftLoad = BandLoad<C, C::VROWS, C::PVC, C::PV>;
+    std::conditional_t<LEFT_DMA, LeftDma, LeftLoad> left_band;
+    BandDma<C, C::NUB, C::RU, C::KBX, C::PU, C::UBAND, 16> right_dma; // (the padding columns of a right row are never read)
+    if constexpr (LEFT_DMA)
+        left_band.init(lane, group, W);
+    else
+        left_band.init(tid, W);
+    right_dma.init(lane, group, W);
 
-    const size_t HW = (size_t)W * H;
-    const int nbv = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
-    const int nbu = u_limit - u_first < C::NUL ? u_limit - u_first : C::NUL;
-
-    // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner). (Fetching the next stage into
-    // registers before the current one is swept, to hide the load latency behind the matrix instructions, measured
-    // 2 % slower on large matrices and no faster on small ones: the other blocks of the CU already cover it.)
-    BandStager<C, C::NVB, C::VROWS, C::PVC, C::PV, C::VBAND> left_stager;
-    BandStager<C, C::NUB, C::RU, C::KBX, C::PU, C::UBAND> right_stager; // (the padding columns of a right row are never read)
-    left_stager.init(tid, W, HW);
-    right_stager.init(tid, W, HW);
-    const T *left_first = g.V + (size_t)v_first * HW, *right_first = g.U + (size_t)u_first * HW;
-    // yl0: the left row of the first copy (the base row yb of the header); the last copy is (JYO - 1) * IY rows ahead of it.
-    // Base rows below syb or from syb + IYB + H - 1 on meet no right row.
-    int yl_begin = clo - (C::JYO - 1) * C::IY, yl_end = chi;
-    if (C::JYO > 1) {
-        if (yl_begin < syb) yl_begin = syb;
-        if (yl_end > syb + C::IYB + H - 1) yl_end = syb + C::IYB + H - 1;
+#ifdef XCORR_EXP_STAGGER
+    if (g.queue != nullptr) {
+        const int phase = (int)(blockIdx.x * 4 / gridDim.x);
+        for (int i = 0; i < phase * XCORR_EXP_STAGGER; ++i) __builtin_amdgcn_s_sleep(32); // 32 x 64 cycles
     }
-    for (int yl0 = yl_begin; yl0 < yl_end; yl0 += C::RL) {
-        for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
-            __syncthreads(); // everyone is done reading the previous stage
-            {
-                // left band: rows [yl0, yl0+VROWS) of the chunk's rows [clo, chi), columns xl = x0 + sxb - shift + col (the 128-bit boundary at or below x0 + sxb)
-                const int xbase = x0 + sxb - left_shift;
-                // right band: rows yr = yl0 - syb - IYB + 1 + row, columns xr = x0 + col
-                const int yr0 = yl0 - syb - C::IYB + 1;
-                const int ur_lo = yr0 < 0 ? -yr0 : 0;
-                const int ur_hi = H - yr0 < C::RU ? H - yr0 : C::RU;
-                const int vr_lo = clo - yl0 > 0 ? clo - yl0 : 0;
-                const int vr_hi = chi - yl0 < C::VROWS ? chi - yl0 : C::VROWS;
-                const int vc_lo = xbase < 0 ? -xbase : 0;
-                const int vc_hi = W - xbase < C::PVC ? W - xbase : C::PVC;
-                const int uc_hi = W - x0 < C::KBX ? W - x0 : C::KBX;
-                left_stager.stage(Vs, left_first + (ptrdiff_t)yl0 * W + xbase, nbv, vr_lo, vr_hi, vc_lo, vc_hi);
-                right_stager.stage(Us, right_first + (ptrdiff_t)yr0 * W + x0, nbu, ur_lo, ur_hi, 0, uc_hi);
-            }
-            __syncthreads();
-            // base rows of this stage whose window of right rows meets the right matrix: yb in [syb, syb + IYB - 1 + H - 1], yb < chi
-            int first = syb - yl0;
-            int last = syb + C::IYB + H - 2 - yl0;
-            if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
-            if (last > C::RL - 1) last = C::RL - 1;
-            const int row0 = first > 0 ? first : 0;
-            const int nrows = last + 1 - row0;
-            // column chunks of this stage that overlap the tile's x shifts: (x0 + kc*K + K-1) + (sxb + TXB-1) >= 0,
-            // (x0 + kc*K) + sxb <= W-1 and x0 + kc*K < w_hi
-            int kc_lo = 0, kc_hi = C::KBX / K;
-            {
-                int need = -(sxb + C::TXB - 1) - (K - 1) - x0;
-                if (need > 0) kc_lo = (need + K - 1) / K;
-                int lim = W - 1 - sxb - x0;
-                if (w_hi - 1 - x0 < lim) lim = w_hi - 1 - x0;
-                int h = lim < 0 ? 0 : lim / K + 1;
-                if (h < kc_hi) kc_hi = h;
-            }
-            if (nrows > 0 && kc_hi > kc_lo) mfma_stage<C>(Vs_lane, Us_lane, acc, group, kc_lo, kc_hi, row0, nrows);
-        }
-    }
+#endif
+    int item = (int)blockIdx.x;
+    for (int turn = 0; item < g.total_items; ++turn) {
+        unsigned fetched = 0;
+        WorkItem wi;
+        const bool something_to_do = decode_work_item<C>(g, item, wi);
+        if (!something_to_do && g.queue != nullptr && tid == 0) fetched = atomicAdd(g.queue, 1u);
+        if (something_to_do) {
+            const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
+            const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
+            // With AL the left bands start at the 128-bit boundary of the matrix rows at or below the tile's first column (x0 is a
+            // multiple of 8): every staged piece is then aligned in global memory and, where the width is a multiple of VK, wholly
+            // inside or outside the matrix; the lanes read `left_shift` columns further in.
+            const int left_shift = ((sxb % VK) + VK) % VK;
+            const T *Vs_lane = Vs_lane0 + left_shift;
 
-    // ---- add the accumulator sets of every result tile, then the partial tiles of the WZ wavefronts through LDS, and write ----
+            acc_t acc[C::TJ][C::TI][C::NC];
 #pragma unroll
-    for (int s = 0; s < C::TJ; ++s)
+            for (int s = 0; s < C::TJ; ++s)
 #pragma unroll
-        for (int t = 0; t < C::TI; ++t)
+                for (int t = 0; t < C::TI; ++t)
 #pragma unroll
-            for (int c = 1; c < C::NC; ++c)
+                    for (int c = 0; c < C::NC; ++c)
 #pragma unroll
-                for (int r = 0; r < C::ACC; ++r) acc[s][t][0][r] += acc[s][t][c][r];
-    // The accumulator elements of a lane are numbered tile * ACC + r and taken in quads of four. In pass q everyone
-    // deposits quads q*QP .. q*QP + QP-1; wavefront w < QP then adds the WZ versions of quad q*QP + w in wavefront order
-    // (deterministic) and writes it: P adjacent x shifts across the lanes.
-    const int Sx = 2 * W - 1, Sy = 2 * H - 1;
-    const size_t out_area = (size_t)Sx * Sy;
-    T *red = reinterpret_cast<T *>(smem_raw);
-    constexpr int PASSES = (C::NQ + C::QP - 1) / C::QP;
+                        for (int r = 0; r < C::ACC; ++r) acc[s][t][c][r] = T(0);
+
+            const int nbv = g.nV - v_first < C::NVB ? g.nV - v_first : C::NVB;
+            const int nbu = u_limit - u_first < C::NUL ? u_limit - u_first : C::NUL;
+            // of the left matrices the rows [clo, chi) of this work item exist, of the right matrices all
+            if constexpr (LEFT_DMA)
+                left_band.set_item(g.V + (size_t)v_first * HW, HW, W, clo, chi - clo, nbv, group);
+            else
+                left_band.set_item(g.V + (size_t)v_first * HW, W, clo, chi - clo, nbv);
+            right_dma.set_item(g.U + (size_t)u_first * HW, HW, W, 0, H, nbu, group);
+
+            // Stages: bands of RL left rows (outer) times blocks of KBX right columns (inner). (Fetching the next stage into
+            // registers before the current one is swept, to hide the load latency behind the matrix instructions, measured
+            // 2 % slower on large matrices and no faster on small ones: the other blocks of the CU already cover it.)
+            // yl0: the left row of the first copy (the base row yb of the header); the last copy is (JYO - 1) * IY rows ahead of it.
+            // Base rows below syb or from syb + IYB + H - 1 on meet no right row.
+            int yl_begin = clo - (C::JYO - 1) * C::IY, yl_end = chi;
+            if (C::JYO > 1) {
+                if (yl_begin < syb) yl_begin = syb;
+                if (yl_end > syb + C::IYB + H - 1) yl_end = syb + C::IYB + H - 1;
+            }
+            for (int yl0 = yl_begin; yl0 < yl_end; yl0 += C::RL) {
+                for (int x0 = xr_lo; x0 < xr_hi; x0 += C::KBX) {
+                    __syncthreads(); // everyone is done reading the previous stage (or adding up the previous item's tiles)
+                    {
+                        // left band: rows [yl0, yl0+VROWS) of the chunk's rows [clo, chi), columns xl = x0 + sxb - shift + col (the 128-bit boundary at or below x0 + sxb)
+                        const int xbase = x0 + sxb - left_shift;
+                        // right band: rows yr = yl0 - syb - IYB + 1 + row, columns xr = x0 + col
+                        const int yr0 = yl0 - syb - C::IYB + 1;
+                        right_dma.stage(Us, W, yr0, x0, lane, group);
+                        if constexpr (LEFT_DMA)
+                            left_band.stage(Vs, W, yl0 - clo, xbase, lane, group);
+                        else
+                            left_band.stage(Vs, W, yl0 - clo, xbase, tid);
+                        dma_wait();
+                        if constexpr (LEFT_DMA) left_band.fix_right_edge(Vs, W, xbase, lane, group);
+                        right_dma.fix_right_edge(Us, W, x0, lane, group);
+                    }
+                    __syncthreads();
+                    // base rows of this stage whose window of right rows meets the right matrix: yb in [syb, syb + IYB - 1 + H - 1], yb < chi
+                    int first = syb - yl0;
+                    int last = syb + C::IYB + H - 2 - yl0;
+                    if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
+                    if (last > C::RL - 1) last = C::RL - 1;
+                    const int row0 = first > 0 ? first : 0;
+                    const int nrows = last + 1 - row0;
+                    // column chunks of this stage that overlap the tile's x shifts: (x0 + kc*K + K-1) + (sxb + TXB-1) >= 0,
+                    // (x0 + kc*K) + sxb <= W-1 and x0 + kc*K < w_hi
+                    int kc_lo = 0, kc_hi = C::KBX / K;
+                    {
+                        int need = -(sxb + C::TXB - 1) - (K - 1) - x0;
+                        if (need > 0) kc_lo = (need + K - 1) / K;
+                        int lim = W - 1 - sxb - x0;
+                        if (w_hi - 1 - x0 < lim) lim = w_hi - 1 - x0;
+                        int h = lim < 0 ? 0 : lim / K + 1;
+                        if (h < kc_hi) kc_hi = h;
+                    }
+                    if (nrows > 0 && kc_hi > kc_lo) {
+                        __builtin_amdgcn_s_setprio(0);
+                        mfma_stage<C>(Vs_lane, Us_lane, acc, group, kc_lo, kc_hi, row0, nrows);
+                        __builtin_amdgcn_s_setprio(2);
+                    }
+                }
+            }
+
+            // ---- add the accumulator sets of every result tile, then the partial tiles of the WZ wavefronts through LDS, and write ----
 #pragma unroll
-    for (int q = 0; q < PASSES; ++q) {
-        __syncthreads(); // the bands, or the previous pass, are no longer read
+            for (int s = 0; s < C::TJ; ++s)
 #pragma unroll
-        for (int o = 0; o < C::QP; ++o) {
-            const int Q = q * C::QP + o;
-            if (Q < C::NQ) {
+                for (int t = 0; t < C::TI; ++t)
+#pragma unroll
+                    for (int c = 1; c < C::NC; ++c)
+#pragma unroll
+                        for (int r = 0; r < C::ACC; ++r) acc[s][t][0][r] += acc[s][t][c][r];
+            // The accumulator elements of a lane are numbered tile * ACC + r and taken in quads of four. In pass q everyone
+            // deposits quads q*QP .. q*QP + QP-1; wavefront w < QP then adds the WZ versions of quad q*QP + w in wavefront order
+            // (deterministic) and writes it: P adjacent x shifts across the lanes.
+            // (the item after this one: asked for here, so that the answer travels while the tiles are added up and written)
+            if (g.queue != nullptr && tid == 0) fetched = atomicAdd(g.queue, 1u);
+            T *red = reinterpret_cast<T *>(smem_raw);
+            constexpr int PASSES = (C::NQ + C::QP - 1) / C::QP;
+#pragma unroll
+            for (int q = 0; q < PASSES; ++q) {
+                __syncthreads(); // the bands, or the previous pass, are no longer read
+#pragma unroll
+                for (int o = 0; o < C::QP; ++o) {
+                    const int Q = q * C::QP + o;
+                    if (Q < C::NQ) {
+                        const int tile = Q * 4 / C::ACC, r0 = Q * 4 % C::ACC;
+                        T *dst = red + ((size_t)(o * C::WZ + group) * 64 + lane) * 4;
+#pragma unroll
+                        for (int e = 0; e < 4; e += VK) {
+                            vec piece;
+#pragma unroll
+                            for (int x = 0; x < VK; ++x) piece[x] = acc[tile / C::TI][tile % C::TI][0][r0 + e + x];
+                            *reinterpret_cast<vec *>(dst + e) = piece;
+                        }
+                    }
+                }
+                __syncthreads();
+                const int Q = q * C::QP + group;
                 const int tile = Q * 4 / C::ACC, r0 = Q * 4 % C::ACC;
-                T *dst = red + ((size_t)(o * C::WZ + group) * 64 + lane) * 4;
+                const int s = tile / C::TI, t = tile % C::TI;
+                const int v = v_first + (s / C::MJX) * C::JV + vj;
+                const int ox = sxb + (s % C::MJX) * C::JX + sxl + (W - 1);
+                if (group < C::QP && Q < C::NQ && v < g.nV && ox >= 0 && ox < Sx) {
+                    T sum[4];
 #pragma unroll
-                for (int e = 0; e < 4; e += VK) {
-                    vec piece;
+                    for (int src = 0; src < C::WZ; ++src) {
+                        const T *from = red + ((size_t)(group * C::WZ + src) * 64 + lane) * 4;
 #pragma unroll
-                    for (int x = 0; x < VK; ++x) piece[x] = acc[tile / C::TI][tile % C::TI][0][r0 + e + x];
-                    *reinterpret_cast<vec *>(dst + e) = piece;
+                        for (int e = 0; e < 4; e += VK) {
+                            vec piece = *reinterpret_cast<const vec *>(from + e);
+#pragma unroll
+                            for (int x = 0; x < VK; ++x) sum[e + x] = src == 0 ? piece[x] : sum[e + x] + piece[x];
+                        }
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int i = C::Op::row(r0 + e, kk); // result row: right matrix, y shift
+                        const int u = u_first + (t / C::NIY) * C::IU + i / C::IY;
+                        const int oy = syb + yo * C::IYB + (t % C::NIY) * C::IY + i % C::IY + (H - 1);
+                        if (u < u_limit && oy >= 0 && oy < Sy) {
+                            const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
+                            T *o = g.out + mat_index * out_area + (size_t)oy * Sx + ox;
+                            if (g.atomic)
+                                atomic_add(o, sum[e]);
+                            else
+                                *o = sum[e];
+                        }
+                    }
                 }
             }
         }
-        __syncthreads();
-        const int Q = q * C::QP + group;
-        const int tile = Q * 4 / C::ACC, r0 = Q * 4 % C::ACC;
-        const int s = tile / C::TI, t = tile % C::TI;
-        const int v = v_first + (s / C::MJX) * C::JV + vj;
-        const int ox = sxb + (s % C::MJX) * C::JX + sxl + (W - 1);
-        if (group < C::QP && Q < C::NQ && v < g.nV && ox >= 0 && ox < Sx) {
-            T sum[4];
-#pragma unroll
-            for (int src = 0; src < C::WZ; ++src) {
-                const T *from = red + ((size_t)(group * C::WZ + src) * 64 + lane) * 4;
-#pragma unroll
-                for (int e = 0; e < 4; e += VK) {
-                    vec piece = *reinterpret_cast<const vec *>(from + e);
-#pragma unroll
-                    for (int x = 0; x < VK; ++x) sum[e + x] = src == 0 ? piece[x] : sum[e + x] + piece[x];
-                }
-            }
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int i = C::Op::row(r0 + e, kk); // result row: right matrix, y shift
-                const int u = u_first + (t / C::NIY) * C::IU + i / C::IY;
-                const int oy = syb + yo * C::IYB + (t % C::NIY) * C::IY + i % C::IY + (H - 1);
-                if (u < u_limit && oy >= 0 && oy < Sy) {
-                    const size_t mat_index = g.group_m > 0 ? (size_t)u : (size_t)v * g.nU + u;
-                    T *o = g.out + mat_index * out_area + (size_t)oy * Sx + ox;
-                    if (g.atomic)
-                        atomic_add(o, sum[e]);
-                    else
-                        *o = sum[e];
-                }
-            }
+        // ---- the next item ----
+        if (g.queue == nullptr) {
+            item += (int)gridDim.x;
+        } else {
+            // (slot `turn & 1`: a wavefront may still read this turn's slot while thread 0, one barrier ahead at most, writes the next turn's)
+            if (tid == 0) handover[turn & 1] = (int)(gridDim.x + fetched);
+            __syncthreads();
+            item = __builtin_amdgcn_readfirstlane(handover[turn & 1]);
+        }
+    }
+    if (g.queue != nullptr && tid == 0) {
+        // The last block to finish zeroes the queue for the next launch that uses it. (Every block's last request precedes its
+        // count here: the request's answer ended its loop.)
+        if (atomicAdd(g.queue + 1, 1u) == gridDim.x - 1) {
+            __hip_atomic_store(g.queue, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(g.queue + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

@@ -16,19 +16,19 @@ using M_64x32 = MfmaCfg<float, 1, 1, 2, 1, 1, 1, 32, 64, 4>;
 using M_32x8_r4 = MfmaCfg<float, 1, 4, 1, 1, 1, 1, 32, 32, 4>;
 // (two result tiles per wavefront: stages of 16 rows and four pieces per staging batch keep them at 128 registers and four blocks per CU,
 // 3-8 % faster than stages of 32 rows at three blocks)
-using M_32x8_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 16, 32, 4, 0, 1, 4, 4>;
+using M_32x8_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 16, 32, 4>;
 // the same right matrices with a square tile of shifts: the columns of a result tile are 16 x shifts twice, 8 left rows apart
-using M_16x16_r4 = MfmaCfg<float, 1, 4, 1, 1, 1, 1, 32, 32, 4, 0, 1, 4, 8, 2>;
-using M_16x16_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 16, 32, 4, 0, 1, 4, 4, 2>;
+using M_16x16_r4 = MfmaCfg<float, 1, 4, 1, 1, 1, 1, 32, 32, 4, 1, 4, 2>;
+using M_16x16_r8 = MfmaCfg<float, 1, 4, 1, 1, 1, 2, 16, 32, 4, 1, 4, 2>;
 // (four copies 4 rows apart with 8 right matrices - 8 x 16 shifts, MfmaCfg<float, 1, 8, 1, 1, 1, 1, 32, 32, 3, 0, 1, 4, 8, 4> - measured
 // 2-8 % behind M_16x16_r4 wherever it ran, its eight right bands leave three blocks per CU: not compiled)
 // ... and rows over right, columns over left matrices (n_to_m)
 // (stages of 16 rows and four pieces per staging batch: 112 registers, four blocks per CU; 32 rows at three blocks 4-10 % slower)
-using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 16, 32, 4, 1, 1, 4, 4>;
+using M_8x8_l4r4 = MfmaCfg<float, 4, 4, 1, 1, 1, 1, 16, 32, 4>;
 // two result tiles per wavefront over eight right matrices: half the work items, each staging 1.5 x the bands for twice the products (128
 // registers, four blocks per CU): 6-16 % faster than the 4 x 4 tile on 16x16 ... 64x64 matrices, level at 128x128. (Eight left matrices instead:
 // 2-4 % behind this one; the fp64 counterparts need 168 registers or 64 KB of LDS and are 8-14 % slower than the fp64 4 x 4 tile: not compiled.)
-using M_8x8_l4r8 = MfmaCfg<float, 4, 4, 1, 1, 1, 2, 16, 32, 4, 1, 1, 4, 4>;
+using M_8x8_l4r8 = MfmaCfg<float, 4, 4, 1, 1, 1, 2, 16, 32, 4>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)

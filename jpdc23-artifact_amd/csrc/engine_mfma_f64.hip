@@ -14,7 +14,7 @@ using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
 // has them - measured level with D_32x8_r4 from 64x64 matrices on and 6 % faster on 32x32 only: not compiled)
 // (stages of 12 rows and four pieces per staging batch: 128 registers and 40 KB of LDS, four blocks per CU; 16 rows at three blocks 2 % slower,
 // 8 rows at four blocks level with that)
-using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4, 1, 1, 4, 4>;
+using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4>;
 
 static const EngineSpec specs[] = {
     make_spec<D_32x32>("f64_m32x32", 0.75, 1.0),

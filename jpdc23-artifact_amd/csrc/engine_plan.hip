@@ -5,6 +5,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "engine_registry.hpp"
 
@@ -409,6 +410,61 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     return shape_plan(*best, rq, rc, xc > 1 ? xc : 1, plan);
 }
 
+// ---- work queues of persistent launches ----
+// A persistent launch (matrix-core sweep, more work items than the device holds blocks) hands out its work items through a
+// counter in device memory. Launches on one stream run one after the other, so every stream gets a counter pair of its own, in
+// a fixed array that belongs to the library's code object (nothing is allocated); a kernel leaves its pair zeroed. Streams
+// that cannot be told apart by their handle (the per-thread default stream) or that are being captured into a graph - whose
+// replays may run beside anything - get no queue: such launches run one block per work item.
+constexpr int QUEUE_SLOTS = 64, QUEUE_STRIDE = 64; // 256 bytes apart: one counter pair per cache line pair
+static __device__ __align__(256) unsigned launch_queues[QUEUE_SLOTS * QUEUE_STRIDE];
+
+struct QueueTable {
+    std::mutex lock;
+    unsigned *base[MAX_DEVICES] = {};
+    hipStream_t owner[MAX_DEVICES][QUEUE_SLOTS] = {};
+    int used[MAX_DEVICES] = {};
+};
+static QueueTable &queue_table() {
+    static QueueTable t;
+    return t;
+}
+
+// The queue of `stream` on the current device, or nullptr if it can have none. Call with the table locked, and keep it locked
+// until the launch that uses the queue has been enqueued (an idle stream's slot may be given to another stream).
+static unsigned *queue_for(hipStream_t stream) {
+    if (stream == hipStreamPerThread) return nullptr;
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return nullptr;
+    }
+    QueueTable &t = queue_table();
+    const int dev = current_device();
+    if (t.base[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(launch_queues)) != hipSuccess || p == nullptr) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        t.base[dev] = static_cast<unsigned *>(p);
+    }
+    for (int i = 0; i < t.used[dev]; ++i)
+        if (t.owner[dev][i] == stream) return t.base[dev] + (size_t)i * QUEUE_STRIDE;
+    if (t.used[dev] < QUEUE_SLOTS) {
+        t.owner[dev][t.used[dev]] = stream;
+        return t.base[dev] + (size_t)(t.used[dev]++) * QUEUE_STRIDE;
+    }
+    // all slots taken: one whose stream has no work in flight (or no longer exists) can change hands
+    for (int i = 0; i < QUEUE_SLOTS; ++i)
+        if (hipStreamQuery(t.owner[dev][i]) != hipErrorNotReady) {
+            (void)hipGetLastError();
+            t.owner[dev][i] = stream;
+            return t.base[dev] + (size_t)i * QUEUE_STRIDE;
+        }
+    return nullptr;
+}
+
 template <typename T>
 static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStream_t stream) {
     EngineArgs<T> a;
@@ -431,12 +487,21 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     a.total_items = plan.total_items;
     a.x_chunks = plan.x_chunks;
     a.x_chunk_cols = plan.x_chunk_cols;
+    a.queue = nullptr;
     if (plan.zero_fill) {
         size_t n = (size_t)(2 * rq.W - 1) * (2 * rq.H - 1) * (rq.group_m > 0 ? (size_t)rq.nU : (size_t)rq.nV * rq.nU);
         size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
         if (blocks > 65536) blocks = 65536;
         zero_fill_kernel<T><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a.out, n);
         XCORR_HIP(hipGetLastError());
+    }
+    // more work items than the device holds blocks of this kernel: as many blocks as it holds, fed from the stream's queue
+    const long slots = (long)device_cus() * plan.spec->resident_blocks();
+    if (plan.spec->MFMA && plan.total_items > slots) {
+        std::lock_guard<std::mutex> guard(queue_table().lock);
+        a.queue = queue_for(stream);
+        XCORR_HIP(plan.spec->launch(&a, a.queue ? (unsigned)slots : plan.grid, stream));
+        return XCORR_OK;
     }
     XCORR_HIP(plan.spec->launch(&a, plan.grid, stream));
     return XCORR_OK;

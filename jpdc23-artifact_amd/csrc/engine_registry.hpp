@@ -7,6 +7,7 @@
 // geometry actually used is reported through xcorr_last_launch().
 #pragma once
 
+#include <cstdlib>
 #include "engine.hpp"
 #include "engine_mfma.hpp"
 #include "xcorr_common.hpp"
@@ -50,9 +51,16 @@ constexpr auto kernel_of() {
         return &engine_kernel<C>;
 }
 
+// EXPERIMENT: dynamic LDS size override
+template <class C>
+int exp_lds() {
+    static int v = -1;
+    if (v < 0) { const char *e = getenv("XCORR_EXP_LDS"); v = e ? atoi(e) : 0; }
+    return C::MFMA && v > C::LDS_BYTES ? v : C::LDS_BYTES;
+}
 template <class C>
 hipError_t allow_large_lds() {
-    if (C::LDS_BYTES <= 64 * 1024) return hipSuccess;
+    if (exp_lds<C>() <= 64 * 1024) return hipSuccess;
     // the attribute belongs to the kernel's copy on one device: kept per device of the process
     static bool attr_set[64] = {};
     int dev = 0;
@@ -60,7 +68,7 @@ hipError_t allow_large_lds() {
     const bool tracked = dev >= 0 && dev < 64;
     if (!tracked || !attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel_of<C>()),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, exp_lds<C>());
         if (e != hipSuccess) return e;
         if (tracked) attr_set[dev] = true;
     }
@@ -71,7 +79,7 @@ template <class C>
 hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
     using T = typename C::value_type;
     if (hipError_t e = allow_large_lds<C>(); e != hipSuccess) return e;
-    kernel_of<C>()<<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
+    kernel_of<C>()<<<dim3(grid), dim3(C::NT), exp_lds<C>(), stream>>>(*static_cast<const EngineArgs<T> *>(args));
     return hipGetLastError();
 }
 
@@ -82,7 +90,7 @@ int resident_blocks_engine() {
     if (blocks[dev] == 0) {
         int n = 0;
         if (allow_large_lds<C>() != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, exp_lds<C>()) != hipSuccess || n < 1) {
             (void)hipGetLastError();
             n = 1;
         }
