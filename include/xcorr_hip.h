@@ -87,6 +87,11 @@ extern "C" {
  * further down select a tile exactly.
  */
 typedef struct xcorr_params {
+    unsigned struct_size;                    /* sizeof(xcorr_params) as the CALLER's header declares it (XCORR_PARAMS_INIT sets it).
+                                                The library reads that many bytes and takes fields it knows beyond them as 0, so a
+                                                caller built against an older header keeps working when fields are appended; 0 is
+                                                rejected (a struct laid out before this field existed starts with
+                                                warps_per_thread_block, usually 0) */
     unsigned warps_per_thread_block;         /* <= 32 */
     unsigned shifts_per_thread_block;        /* <= 32, warp-per-overlap family */
     unsigned rows_per_thread;                /* split-row contract: max overlap rows per worker (JSON rows_per_thread / rows_per_warp);
@@ -121,6 +126,8 @@ typedef struct xcorr_params {
                                                 under their own contract when no tile geometry and no chunk below 16 rows is named
                                                 and the launch is large enough; no counterpart in the reference */
 } xcorr_params;
+/* xcorr_params p = XCORR_PARAMS_INIT;  - every tuning field 0 (the library's choice), struct_size set */
+#define XCORR_PARAMS_INIT {sizeof(xcorr_params)}
 
 /* Geometry of the most recent launch (reference kernel_args.hpp:9-33 plus the
  * template parameters each launcher records, e.g. naive_shuffle_multirow_both.cu:488-522). */
@@ -165,7 +172,9 @@ const char *xcorr_version(void);
 /* Planning without launching (per host thread; no counterpart in the reference): while on, the entry points of the
  * sliding-window engine (xcorr_shuffle ... xcorr_multimat_both_grouped) validate their arguments, choose kernel and
  * geometry, fill the launch record and return without launching or reading the pointers. Works without a GPU (256
- * CUs are assumed then); for tools and tests that ask what a call would run. */
+ * CUs and the occupancies of an MI355X are assumed then); for tools and tests that ask what a call would run.
+ * on = 2 plans as if `out` were memory the floating-point atomic add is not defined on (host-mapped, managed): a launch
+ * that would split by the launcher's own choice stays whole, one whose contract is atomic adds is refused. */
 int xcorr_plan_only(int on);
 
 /* ---- memory / queue shims: the C++ host never includes the HIP headers.

@@ -30,6 +30,7 @@ class XcorrError(RuntimeError):
 
 class Params(ctypes.Structure):
     _fields_ = [
+        ("struct_size", ctypes.c_uint),
         ("warps_per_thread_block", ctypes.c_uint),
         ("shifts_per_thread_block", ctypes.c_uint),
         ("rows_per_thread", ctypes.c_uint),
@@ -258,6 +259,7 @@ class Graph:
 
 def make_params(**kw):
     p = Params()
+    p.struct_size = ctypes.sizeof(Params)
     for k, v in kw.items():
         if k == "distribution_type" and isinstance(v, str):
             v = DIST[v]

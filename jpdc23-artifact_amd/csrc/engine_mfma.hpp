@@ -480,15 +480,27 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
         for (int i = 0; i < phase * XCORR_EXP_STAGGER; ++i) __builtin_amdgcn_s_sleep(32); // 32 x 64 cycles
     }
 #endif
+    // The queue this block draws from; the k-th draw stands for item my_queue + gridDim.x + queues * k. (Letting a block whose
+    // queue is empty draw from the others was measured: every block then ends with up to eight draws nothing hides, and all
+    // five benchmark workloads ran 1-2 % slower.)
+    const int my_queue = g.queue != nullptr ? (int)(blockIdx.x % (unsigned)g.queues) : 0;
+    unsigned *const queue = g.queue != nullptr ? g.queue + 32 * my_queue : nullptr;
+    auto next_item = [&](unsigned drawn) __attribute__((always_inline)) { return (int)(my_queue + gridDim.x + (unsigned)g.queues * drawn); };
     int item = (int)blockIdx.x;
     for (int turn = 0; item < g.total_items; ++turn) {
+        // The item after this one is asked for when the last bands of this one have arrived (the answer of the contended counter
+        // takes several times as long as a band, and every wait for bands would be a wait for it as well: it travels during the
+        // last sweep) and is handed to the block before the barrier of the in-block reduction (slot `turn & 1`: a wavefront may
+        // still read this turn's slot while thread 0, one barrier ahead at most, writes the next turn's).
         unsigned fetched = 0;
         WorkItem wi;
         const bool something_to_do = decode_work_item<C>(g, item, wi);
-        if (!something_to_do && g.queue != nullptr && tid == 0) fetched = atomicAdd(g.queue, 1u);
         if (something_to_do) {
-            const int clo = wi.clo, chi = wi.chi, syb = wi.syb, sxb = wi.sxb, v_first = wi.v_first, u_first = wi.u_first, u_limit = wi.u_limit;
-            const int xr_lo = wi.xr_lo, xr_hi = wi.xr_hi, w_hi = wi.w_hi;
+            // (the same for all threads; said so that everything derived from them - loop bounds, buffer descriptors - stays in scalar registers)
+            auto uniform = [](int x) __attribute__((always_inline)) { return __builtin_amdgcn_readfirstlane(x); };
+            const int clo = uniform(wi.clo), chi = uniform(wi.chi), syb = uniform(wi.syb), sxb = uniform(wi.sxb), v_first = uniform(wi.v_first),
+                      u_first = uniform(wi.u_first), u_limit = uniform(wi.u_limit);
+            const int xr_lo = uniform(wi.xr_lo), xr_hi = uniform(wi.xr_hi), w_hi = uniform(wi.w_hi);
             // With AL the left bands start at the 128-bit boundary of the matrix rows at or below the tile's first column (x0 is a
             // multiple of 8): every staged piece is then aligned in global memory and, where the width is a multiple of VK, wholly
             // inside or outside the matrix; the lanes read `left_shift` columns further in.
@@ -542,6 +554,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
                         right_dma.fix_right_edge(Us, W, x0, lane, group);
                     }
                     __syncthreads();
+                    if (yl0 + C::RL >= yl_end && x0 + C::KBX >= xr_hi && g.queue != nullptr && tid == 0) fetched = atomicAdd(queue, 1u);
                     // base rows of this stage whose window of right rows meets the right matrix: yb in [syb, syb + IYB - 1 + H - 1], yb < chi
                     int first = syb - yl0;
                     int last = syb + C::IYB + H - 2 - yl0;
@@ -580,8 +593,7 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
             // The accumulator elements of a lane are numbered tile * ACC + r and taken in quads of four. In pass q everyone
             // deposits quads q*QP .. q*QP + QP-1; wavefront w < QP then adds the WZ versions of quad q*QP + w in wavefront order
             // (deterministic) and writes it: P adjacent x shifts across the lanes.
-            // (the item after this one: asked for here, so that the answer travels while the tiles are added up and written)
-            if (g.queue != nullptr && tid == 0) fetched = atomicAdd(g.queue, 1u);
+            if (g.queue != nullptr && tid == 0) handover[turn & 1] = next_item(fetched);
             T *red = reinterpret_cast<T *>(smem_raw);
             constexpr int PASSES = (C::NQ + C::QP - 1) / C::QP;
 #pragma unroll
@@ -641,18 +653,19 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
         if (g.queue == nullptr) {
             item += (int)gridDim.x;
         } else {
-            // (slot `turn & 1`: a wavefront may still read this turn's slot while thread 0, one barrier ahead at most, writes the next turn's)
-            if (tid == 0) handover[turn & 1] = (int)(gridDim.x + fetched);
-            __syncthreads();
+            if (!something_to_do) {
+                if (tid == 0) handover[turn & 1] = next_item(atomicAdd(queue, 1u));
+                __syncthreads();
+            }
             item = __builtin_amdgcn_readfirstlane(handover[turn & 1]);
         }
     }
-    if (g.queue != nullptr && tid == 0) {
-        // The last block to finish zeroes the queue for the next launch that uses it. (Every block's last request precedes its
-        // count here: the request's answer ended its loop.)
-        if (atomicAdd(g.queue + 1, 1u) == gridDim.x - 1) {
-            __hip_atomic_store(g.queue, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(g.queue + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (queue != nullptr && tid == 0) {
+        // The last block of a queue to finish zeroes it for the next launch that uses it. (Every block's last draw precedes its
+        // count here: the draw's answer ended its loop. gridDim.x is a multiple of the number of queues.)
+        if (atomicAdd(queue + 1, 1u) == gridDim.x / (unsigned)g.queues - 1) {
+            __hip_atomic_store(queue, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(queue + 1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
 }

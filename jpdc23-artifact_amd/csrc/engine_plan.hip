@@ -191,6 +191,24 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     const double per_block = (fixed + t_stage * stages_avg) / n1 + inst_avg * cyc / e_full;
     const double tail = k_tail * crit;
     double t = std::fmax(items * per_block / cus + tail, crit);
+    if (s.MFMA) {
+        // The matrix-core kernel runs `slots` persistent blocks that take the items in launch order, heaviest first: the launch
+        // is a number of full rounds of items that share their CU with occ - 1 others, a last, partly filled round of small items
+        // with fewer neighbours, and the difference between the first round's items and the average ones.
+        const double k_last = 0.6;
+        auto item_time = [&](double inst, double stages, double n) {
+            return fixed + t_stage * stages + n * inst * cyc / (e_full * (1.0 - std::exp(-n / tau)));
+        };
+        const double slots = (double)cus * occ;
+        if (items <= slots) {
+            t = item_time(inst_max, stages_max, n1);
+        } else {
+            const double full = std::floor(items / slots), rest = items - full * slots;
+            const double n_last = std::fmax(1.0, std::fmin((double)occ, std::ceil(rest / cus)));
+            t = full * item_time(inst_avg, stages_avg, occ) + (rest > 0 ? item_time(inst_avg * k_last, stages_avg, n_last) : 0.0) +
+                k_tail * (item_time(inst_max, stages_max, occ) - item_time(inst_avg, stages_avg, occ));
+        }
+    }
     if (split) t += t_clear + items * 64.0 * s.NV * s.NU * s.A * s.B * us_per_atomic;
     // Sustained vector-FMA load pulls the power-managed shader clock from 2.35 to 2.0-2.1 GHz within the first milliseconds
     // of a launch (random operands); the matrix cores hold 2.35 GHz on the same data. Measured / predicted run time of the
@@ -416,7 +434,7 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
 // a fixed array that belongs to the library's code object (nothing is allocated); a kernel leaves its pair zeroed. Streams
 // that cannot be told apart by their handle (the per-thread default stream) or that are being captured into a graph - whose
 // replays may run beside anything - get no queue: such launches run one block per work item.
-constexpr int QUEUE_SLOTS = 64, QUEUE_STRIDE = 64; // 256 bytes apart: one counter pair per cache line pair
+constexpr int QUEUE_SLOTS = 64, QUEUES = 8, QUEUE_STRIDE = 32 * QUEUES; // per stream: eight counter pairs, 128 bytes apart
 static __device__ __align__(256) unsigned launch_queues[QUEUE_SLOTS * QUEUE_STRIDE];
 
 struct QueueTable {
@@ -488,6 +506,7 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     a.x_chunks = plan.x_chunks;
     a.x_chunk_cols = plan.x_chunk_cols;
     a.queue = nullptr;
+    a.queues = 1;
     if (plan.zero_fill) {
         size_t n = (size_t)(2 * rq.W - 1) * (2 * rq.H - 1) * (rq.group_m > 0 ? (size_t)rq.nU : (size_t)rq.nV * rq.nU);
         size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
@@ -500,6 +519,7 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     if (plan.spec->MFMA && plan.total_items > slots) {
         std::lock_guard<std::mutex> guard(queue_table().lock);
         a.queue = queue_for(stream);
+        a.queues = slots % QUEUES == 0 ? QUEUES : 1;
         XCORR_HIP(plan.spec->launch(&a, a.queue ? (unsigned)slots : plan.grid, stream));
         return XCORR_OK;
     }
@@ -540,10 +560,37 @@ static int cached_plan(const EngineRequest &rq, EnginePlan &plan) {
     return XCORR_OK;
 }
 
-int run_engine(const EngineRequest &rq, hipStream_t stream) {
+// The hardware's floating-point atomic add is only defined on ordinary (coarse-grained) device memory; on host-mapped or managed
+// allocations it is dropped without an error. True if `out` is memory a split plan may accumulate into. The answer for the
+// last pointer asked about is kept per thread (a query costs about a microsecond).
+static bool atomics_defined_on(const void *out) {
+    if (plan_only()) return plan_only_mode() != 2;
+    thread_local const void *last = nullptr;
+    thread_local bool last_ok = false;
+    if (out == last && out != nullptr) return last_ok;
+    hipPointerAttribute_t attr;
+    bool ok = hipPointerGetAttributes(&attr, out) == hipSuccess && attr.type == hipMemoryTypeDevice && !attr.isManaged;
+    (void)hipGetLastError();
+    last = out;
+    last_ok = ok;
+    return ok;
+}
+
+int run_engine(const EngineRequest &request, hipStream_t stream) {
+    EngineRequest rq = request;
     EnginePlan plan;
     int rc = cached_plan(rq, plan);
     if (rc != XCORR_OK) return rc;
+    if (plan.atomic && !atomics_defined_on(rq.out)) {
+        if (rq.caller_zeroes || !rq.may_split || rq.rows_per_worker != 0 || rq.column_chunks > 1)
+            return fail(XCORR_ERR_UNSUPPORTED,
+                        "%s: this launch adds partial sums with floating-point atomics, which are only defined on ordinary device memory "
+                        "(hipMalloc); `out` is host-mapped, managed or unknown memory", rq.family);
+        // the launcher's own choice to split: the whole reduction per work item instead, plain stores
+        rq.may_split = false;
+        rq.column_chunks = 1;
+        if ((rc = cached_plan(rq, plan)) != XCORR_OK) return rc;
+    }
     if (!plan_only()) {
         rc = rq.elem_bytes == 4 ? launch_typed<float>(rq, plan, stream) : launch_typed<double>(rq, plan, stream);
         if (rc != XCORR_OK) return rc;

@@ -19,7 +19,7 @@ extern "C" {
 // ------------------------------------------------------------------ status
 const char *xcorr_last_error(void) { return error_buffer(); }
 
-const char *xcorr_version(void) { return "xcorr_hip 0.1 (gfx950)"; }
+const char *xcorr_version(void) { return "xcorr_hip 0.2 (gfx950)"; }
 
 int xcorr_last_launch(xcorr_launch_record *out) {
     if (!out) return fail(XCORR_ERR_INVALID_ARGUMENT, "null record pointer");
@@ -29,7 +29,9 @@ int xcorr_last_launch(xcorr_launch_record *out) {
 }
 
 int xcorr_plan_only(int on) {
+    if (on < 0 || on > 2) return fail(XCORR_ERR_INVALID_ARGUMENT, "xcorr_plan_only: %d is not 0, 1 or 2", on);
     plan_only() = on != 0;
+    plan_only_mode() = on;
     return XCORR_OK;
 }
 
@@ -193,9 +195,24 @@ int xcorr_event_destroy(void *event) {
 // ------------------------------------------------------------------ compute
 namespace {
 
-const xcorr_params zero_params = {};
-
-const xcorr_params &params_or_default(const xcorr_params *p) { return p ? *p : zero_params; }
+// The caller's parameter block, as much of it as the caller's header declares (struct_size), in the layout of this build;
+// a null pointer stands for all defaults.
+struct LoadedParams {
+    xcorr_params p = {};
+    int error = XCORR_OK;
+    explicit LoadedParams(const xcorr_params *from) {
+        p.struct_size = sizeof(xcorr_params);
+        if (!from) return;
+        const unsigned n = from->struct_size;
+        if (n < 2 * sizeof(unsigned) || n % sizeof(unsigned) != 0) {
+            error = fail(XCORR_ERR_INVALID_ARGUMENT,
+                         "xcorr_params.struct_size is %u: set it to sizeof(xcorr_params) (XCORR_PARAMS_INIT; the field leads the struct since version 0.2)", n);
+            return;
+        }
+        memcpy(&p, from, n < sizeof(xcorr_params) ? n : sizeof(xcorr_params));
+        p.struct_size = sizeof(xcorr_params);
+    }
+};
 
 int check_dist(unsigned d) {
     if (d > XCORR_DIST_TRIANGLE) return fail(XCORR_ERR_INVALID_ARGUMENT, "Unknown distribution %u", d);
@@ -231,7 +248,9 @@ EngineRequest base_request(const char *family, int elem_bytes, const void *left,
 template <typename T>
 int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
                  void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
@@ -249,7 +268,9 @@ int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
 template <typename T>
 int split_row_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
                    void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
@@ -265,7 +286,9 @@ int split_row_impl(const T *left, const T *right, T *out, unsigned cols, unsigne
 template <typename T>
 int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
                  void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
@@ -294,7 +317,9 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
 template <typename T>
 int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left, unsigned n_right,
                         const xcorr_params *pp, void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_counts(n_left, n_right, n_left > 1))) return rc;
@@ -320,7 +345,9 @@ int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, un
 template <typename T>
 int multimat_right_grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
                                 unsigned n_right, const xcorr_params *pp, void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_counts(n_left, n_right, true))) return rc;
@@ -344,7 +371,9 @@ int multimat_right_grouped_impl(const T *left, const T *right, T *out, unsigned 
 template <typename T>
 int multimat_both_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
                        unsigned n_right, const xcorr_params *pp, void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_counts(n_left, n_right, true))) return rc;
@@ -365,7 +394,9 @@ int multimat_both_impl(const T *left, const T *right, T *out, unsigned cols, uns
 template <typename T>
 int multimat_both_grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_left,
                                unsigned n_right, const xcorr_params *pp, void *stream) {
-    const xcorr_params &p = params_or_default(pp);
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_counts(n_left, n_right, true))) return rc;
@@ -407,29 +438,41 @@ int xcorr_overlap_wise_all_pairs_f64(const double *left, const double *right, do
 
 int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                                const xcorr_params *p, void *stream) {
-    return run_warp_per_overlap<float>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_warp_per_overlap<float>(left, right, out, cols, rows, loaded.p, as_stream(stream));
 }
 int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                const xcorr_params *p, void *stream) {
-    return run_warp_per_overlap<double>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_warp_per_overlap<double>(left, right, out, cols, rows, loaded.p, as_stream(stream));
 }
 
 int xcorr_warp_per_overlap_lds_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                                    unsigned n_right, const xcorr_params *p, void *stream) {
-    return run_warp_per_overlap_lds<float>(left, right, out, cols, rows, n_right, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_warp_per_overlap_lds<float>(left, right, out, cols, rows, n_right, loaded.p, as_stream(stream));
 }
 int xcorr_warp_per_overlap_lds_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                    unsigned n_right, const xcorr_params *p, void *stream) {
-    return run_warp_per_overlap_lds<double>(left, right, out, cols, rows, n_right, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_warp_per_overlap_lds<double>(left, right, out, cols, rows, n_right, loaded.p, as_stream(stream));
 }
 
 int xcorr_block_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                                 const xcorr_params *p, void *stream) {
-    return run_block_per_overlap<float>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_block_per_overlap<float>(left, right, out, cols, rows, loaded.p, as_stream(stream));
 }
 int xcorr_block_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                 const xcorr_params *p, void *stream) {
-    return run_block_per_overlap<double>(left, right, out, cols, rows, params_or_default(p), as_stream(stream));
+    const LoadedParams loaded(p);
+    if (loaded.error) return loaded.error;
+    return run_block_per_overlap<double>(left, right, out, cols, rows, loaded.p, as_stream(stream));
 }
 
 #define XCORR_PAIR_ENTRY(NAME, IMPL)                                                                              \

@@ -50,6 +50,11 @@ inline bool &plan_only() {
     static thread_local bool on = false;
     return on;
 }
+// 1: plan as for ordinary device memory; 2: plan as for an output the hardware's float atomics are not defined on
+inline int &plan_only_mode() {
+    static thread_local int mode = 0;
+    return mode;
+}
 inline bool &have_last_launch() {
     static thread_local bool have = false;
     return have;

@@ -252,7 +252,7 @@ protected:
 
 private:
     algorithm_def def_;
-    xcorr_params params_{};
+    xcorr_params params_ = XCORR_PARAMS_INIT;
     bool zero_output_ = false; // clear the output inside the measured block (split-row contract, column groups)
     properties props_;
     unsigned num_streams_ = 0;

@@ -130,3 +130,83 @@ def test_fft_normalize_matches_the_definition():
         s = (2 * rows, 2 * cols)
         raw = np.fft.irfft2(np.fft.rfft2(a, s=s) * np.conj(np.fft.rfft2(b, s=s)), s=s) * (4 * rows * cols)
         assert np.allclose(fft.normalize(raw[None])[0], correlate2d(a, b, mode="full"), atol=1e-12)
+
+
+def test_params_struct_size_rules():
+    """xcorr_params.struct_size: 0 (a struct laid out before the field existed) is refused; a smaller size than this build's
+    (a caller built against an older header) is read that far and the rest taken as 0, whatever lies behind it."""
+    xc = load_package()
+    lib = xc.lib()
+    assert b"0.2" in lib.xcorr_version()
+    dummy = ctypes.c_void_p(16)
+    assert lib.xcorr_plan_only(1) == 0
+    try:
+        p = xc.Params()  # struct_size 0
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 1
+        assert b"struct_size" in lib.xcorr_last_error()
+        p = xc.make_params()
+        assert p.struct_size == ctypes.sizeof(xc.Params)
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 0
+        whole = xc.last_launch()
+        # an older caller: its struct ends before matrix_cores, and what follows in memory is not the library's to read
+        p = xc.make_params(matrix_cores=7)
+        p.struct_size = xc.Params.matrix_cores.offset
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 0, lib.xcorr_last_error()
+        assert xc.last_launch() == whole
+        p.struct_size = ctypes.sizeof(xc.Params)
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 1
+        assert b"matrix_cores" in lib.xcorr_last_error()
+        # a larger struct than this build knows (a newer caller): the known part is read
+        p = xc.make_params(shifts_per_thread=4)
+        p.struct_size = ctypes.sizeof(xc.Params) + 16
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 0
+        assert xc.last_launch()["y_shifts_per_thread"] == 4
+        p.struct_size = 6
+        assert lib.xcorr_grouped_overlap_f32(dummy, dummy, dummy, 200, 200, ctypes.byref(p), None) == 1
+    finally:
+        lib.xcorr_plan_only(0)
+
+
+def test_split_plans_need_ordinary_device_memory():
+    """Plan-only mode 2 plans for an output the float atomic add is not defined on (host-mapped, managed): the launcher's own
+    split is given up for the whole reduction per work item, a contract of atomic adds is refused."""
+    xc = load_package()
+    lib = xc.lib()
+    dummy = ctypes.c_void_p(16)
+
+    def ask(fn, mode, *args, **kw):
+        assert lib.xcorr_plan_only(mode) == 0
+        try:
+            p = xc.make_params(**kw)
+            code = getattr(lib, fn)(dummy, dummy, dummy, *args, ctypes.byref(p), None)
+            return code, (xc.last_launch() if code == 0 else lib.xcorr_last_error())
+        finally:
+            lib.xcorr_plan_only(0)
+
+    code, rec = ask("xcorr_grouped_overlap_f32", 1, 512, 512)
+    assert code == 0 and rec["uses_atomics"] == 1
+    code, rec = ask("xcorr_grouped_overlap_f32", 2, 512, 512)
+    assert code == 0 and rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 512
+    code, rec = ask("xcorr_shuffle_f32", 2, 64, 64, matrix_cores=2)
+    assert code == 0 and rec["uses_atomics"] == 0
+    code, msg = ask("xcorr_split_row_f32", 2, 64, 64)
+    assert code == 3 and b"atomics" in msg
+    code, msg = ask("xcorr_grouped_overlap_f32", 2, 512, 512, rows_per_thread=32)
+    assert code == 3
+    code, rec = ask("xcorr_multimat_both_f64", 2, 32, 32, 4, 4)
+    assert code == 3
+    assert lib.xcorr_plan_only(3) == 1
+
+
+def test_callers_are_told_when_to_zero_the_output():
+    """xcorr_multimat_right with a distribution but no chunk runs under the work-distribution contract (the caller zeroes
+    `out`): the package's own wrapper zeroes in exactly the cases the header names."""
+    xc = load_package()
+    assert not xc.needs_zeroed_output("multimat_right", xc.make_params())
+    assert not xc.needs_zeroed_output("multimat_right", xc.make_params(distribution_type="none"))
+    assert xc.needs_zeroed_output("multimat_right", xc.make_params(distribution_type="rectangle"))
+    assert xc.needs_zeroed_output("multimat_right", xc.make_params(distribution_type="triangle"))
+    assert xc.needs_zeroed_output("multimat_right", xc.make_params(rows_per_thread=4))
+    assert xc.needs_zeroed_output("multimat_right_groups", xc.make_params(rows_per_thread=4))
+    assert xc.needs_zeroed_output("split_row", None) and xc.needs_zeroed_output("multimat_both", None)
+    assert not xc.needs_zeroed_output("grouped_overlap", None) and not xc.needs_zeroed_output("multimat_right_grouped", None)
