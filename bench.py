@@ -22,7 +22,8 @@ from __graft_entry__ import load_oracle, load_package  # noqa: E402
 # MI355X published vector peaks (TFLOP/s)
 PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
 # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs scaled
-# by the library's copy kernel (figures and commands in the profile each entry names). Not measured in this run:
+# by the library's copy kernel (figures and commands in the profile each entry names). Not measured in this run
+# (hardware counters need the profiler around the process): the JSON says so with "traffic_measured_in_run": false.
 # Keyed by (workload, kernel of the launch record): a default launch that picks another tile reports null.
 MEASURED_TRAFFIC = {
     ("C1", "grouped_overlap/pair_in_lds_f32_a1"): (0.32e6 + 0.18e6, "profiles/pair_in_lds_one_to_one_64.md"),
@@ -190,6 +191,40 @@ def single_thread_baseline(oracle, w, budget_s):
     }, picked
 
 
+def parity_against_host_loops(oracle, got0, band, lo, hi, exact, lo64, hi64, dtype):
+    """The three numbers quoted for an fp32 result: relative Frobenius error against the oracle's fp32 host loop (rows [lo, hi)),
+    against the same loop with an fp64 accumulator (rows [lo64, hi64)), and the host loop's own distance from the latter."""
+    bar = 1e-5 if dtype == np.float32 else 1e-12
+    e = oracle.errors(got0[lo:hi], band[lo:hi])
+    out = {
+        "against": f"oracle (fp32 host loop) rows [{lo},{hi}) of pair 0" if dtype == np.float32 else f"oracle rows [{lo},{hi}) of pair 0",
+        "bar": bar,
+        "rel_frobenius": float(f"{e.rel_frobenius:.3e}"),
+        "max_abs": float(f"{e.max_abs:.3e}"),
+        "max_rel": float(f"{e.max_rel:.3e}"),
+        "within_bar_vs_fp32_host_loop" if dtype == np.float32 else "within_bar": bool(e.rel_frobenius <= bar),
+    }
+    if dtype == np.float32:
+        e64 = oracle.errors(got0[lo64:hi64], exact[lo64:hi64])
+        o64 = oracle.errors(band[lo64:hi64], exact[lo64:hi64])
+        out["rows_checked_with_fp64_accumulator"] = [lo64, hi64]
+        out["rel_frobenius_vs_fp64_accumulated"] = float(f"{e64.rel_frobenius:.3e}")
+        out["oracle_fp32_vs_fp64_accumulated"] = float(f"{o64.rel_frobenius:.3e}")
+        out["within_bar_vs_fp64_accumulated"] = bool(e64.rel_frobenius <= bar)
+    return out
+
+
+def timed_variant(xc, workloads, name, family, params_json, steps, warmup):
+    """Another launch of a configuration (family / parameters named by the caller), timed like the headline."""
+    v = Workload(xc, workloads, name, family, params_json)
+    wall, ev = v.timed(steps, warmup)
+    rec = xc.last_launch()
+    entry = roofline_of(v, rec, ev / steps, False)
+    entry.update({"kernel": rec["kernel"], "family": v.family, "params": json.loads(params_json), "steps": steps, "uses_atomics": rec["uses_atomics"],
+                  "rows_per_worker": rec["rows_per_worker"], "ms_per_step": round(wall * 1e3 / steps, 4)})
+    return v, entry
+
+
 def roofline_of(w, rec, kernel_ms, default_launch):
     achieved = w.flop / (kernel_ms * 1e-3) / 1e12
     peak = PEAK_TFLOPS[w.cfg["dtype"]]
@@ -204,6 +239,7 @@ def roofline_of(w, rec, kernel_ms, default_launch):
         "frac": round(achieved / peak, 4),
         "traffic": traffic[0] if traffic else None,
         "traffic_source": traffic[1] if traffic else None,
+        "traffic_measured_in_run": False,
         "algorithmic_bytes": w.algorithmic_bytes,
         "kernel_ms": round(kernel_ms, 4),
     }
@@ -352,28 +388,15 @@ def main():
         single, _ = single_thread_baseline(oracle, w, budget_s=4.0)
         result["cpu_baseline"]["single_thread"] = single
         got = w.d_out.to_numpy(w.out_shape, dtype)
-        e = oracle.errors(got[0][lo:hi], band[lo:hi])
-        bar = 1e-5 if dtype == np.float32 else 1e-12
-        result["parity"] = {
-            "against": f"oracle (fp32 host loop) rows [{lo},{hi}) of pair 0" if dtype == np.float32 else f"oracle rows [{lo},{hi}) of pair 0",
-            "bar": bar,
-            "rel_frobenius": float(f"{e.rel_frobenius:.3e}"),
-            "max_abs": float(f"{e.max_abs:.3e}"),
-            "max_rel": float(f"{e.max_rel:.3e}"),
-            "within_bar_vs_fp32_host_loop" if dtype == np.float32 else "within_bar": bool(e.rel_frobenius <= bar),
-        }
+        exact, lo64, hi64 = None, lo, hi
         if dtype == np.float32:
             # the host loop adds every overlap one product at a time in fp32 and drifts from the exact
             # sum on long overlaps; the same loop with an fp64 accumulator tells the two apart
             mid = (lo + hi) // 2
             lo64, hi64 = max(lo, mid - 8), min(hi, mid + 8)
             exact = oracle.cross_corr(w.left[0], w.right[0], threads=base["cores"], row_begin=lo64, row_end=hi64, acc64=True)
-            e64 = oracle.errors(got[0][lo64:hi64], exact[lo64:hi64])
-            o64 = oracle.errors(band[lo64:hi64], exact[lo64:hi64])
-            result["parity"]["rows_checked_with_fp64_accumulator"] = [lo64, hi64]
-            result["parity"]["rel_frobenius_vs_fp64_accumulated"] = float(f"{e64.rel_frobenius:.3e}")
-            result["parity"]["oracle_fp32_vs_fp64_accumulated"] = float(f"{o64.rel_frobenius:.3e}")
-            result["parity"]["within_bar_vs_fp64_accumulated"] = bool(e64.rel_frobenius <= bar)
+        result["parity"] = parity_against_host_loops(oracle, got[0], band, lo, hi, exact, lo64, hi64, dtype)
+        result["config"]["parity"] = {k: result["parity"][k] for k in result["parity"] if k.startswith("within_bar") or k.startswith("rel_frobenius")}
     w.free()
 
     if args.config == "C2" and default_launch and not args.only and args.data == "config":
@@ -412,6 +435,22 @@ def main():
                                    "max_abs": float(f"{e.max_abs:.3e}"), "within_bar": bool(e.rel_frobenius <= bar)}
             per[name] = entry
             o.free()
+        # The register tiles (vector FMAs) of every configuration, as xcorr_params.matrix_cores = 2 selects them: the fraction of the
+        # VECTOR-FMA roofline next to the default launch's (the matrix cores have the same fp32 / fp64 peak on this chip).
+        for name in ("C2", "C3", "C4", "C5"):
+            v, entry = timed_variant(xc, workloads, name, None, '{"matrix_cores": 2}', 5, 1)
+            v.free()
+            (result if name == "C2" else per[name])["vector_fma_tiles"] = {k: entry[k] for k in ("kernel", "kernel_ms", "achieved", "frac", "bound", "steps")}
+        # C2 launched two more ways: every accumulator running over its whole overlap like a thread of the reference's kernels
+        # (xcorr_shuffle, distribution_type none: the launch that meets the 1e-5 bar against the fp32 host loop), and the
+        # grouped launch without atomic adds (whole reductions per work item: the same bits every run).
+        variants = {"C2_strict": ("shuffle", '{"distribution_type": 1}', 3), "C2_no_atomics": ("grouped_overlap", '{"rows_per_thread": 1024, "column_chunks": 1}', 5)}
+        for key, (family, params_json, steps) in variants.items():
+            v, entry = timed_variant(xc, workloads, "C2", family, params_json, steps, 1)
+            if oracle is not None:
+                entry["parity"] = parity_against_host_loops(oracle, v.d_out.to_numpy(v.out_shape, dtype)[0], band, lo, hi, exact, lo64, hi64, dtype)
+            v.free()
+            per[key] = entry
         result["per_config"] = per
     print(json.dumps(result))
 

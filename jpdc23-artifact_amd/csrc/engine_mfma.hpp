@@ -224,7 +224,7 @@ struct BandDma {
     // Stage whose image row 0, column 0 is row `row0` (relative to row_lo of set_item), column `col0` of the matrices.
     template <bool CHECK>
     __device__ __forceinline__ void copy(T *lds, int W, int row0, int col0, int lane, int wave) const {
-        const unsigned origin = (unsigned)((row0 * W + col0) * EB);
+        const unsigned origin = (unsigned)(((long long)row0 * W + col0) * EB); // (modulo 2^32: a matrix has at most 2^31 bytes)
 #pragma unroll
         for (int i = 0; i < NBW; ++i) {
             T *band = lds + (OWN ? wave + i * C::WZ : 0) * BAND;
@@ -305,7 +305,7 @@ struct BandLoad {
     __device__ __forceinline__ void copy(T *lds, int W, int row0, int col0, int tid) const {
         typedef unsigned uvec __attribute__((ext_vector_type(4)));
         typedef T half_t __attribute__((ext_vector_type(VK / 2)));
-        const unsigned origin = (unsigned)((row0 * W + col0) * EB);
+        const unsigned origin = (unsigned)(((long long)row0 * W + col0) * EB); // (modulo 2^32: a matrix has at most 2^31 bytes)
         uvec val[ITER];
 #pragma unroll
         for (int i = 0; i < ITER; ++i) {

@@ -32,14 +32,14 @@ using M_8x8_l4r8 = MfmaCfg<float, 4, 4, 1, 1, 1, 2, 16, 32, 4>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)
-    make_spec<M_32x32>("f32_m32x32", 0.82, 1.0),
-    make_spec<M_64x32>("f32_m64x32", 0.82, 1.0),
-    make_spec<M_32x8_r4>("f32_m32x8_r4", 0.82, 1.0),
-    make_spec<M_32x8_r8>("f32_m32x8_r8", 0.84, 1.0),
-    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.90, 1.0),
-    make_spec<M_16x16_r4>("f32_m16x16_r4", 0.83, 1.0),
-    make_spec<M_16x16_r8>("f32_m16x16_r8", 0.85, 1.0),
-    make_spec<M_8x8_l4r8>("f32_m8x8_l4r8", 0.89, 1.0),
+    make_spec<M_32x32>("f32_m32x32", 0.716, 1.0),
+    make_spec<M_64x32>("f32_m64x32", 0.749, 1.0),
+    make_spec<M_32x8_r4>("f32_m32x8_r4", 0.707, 1.0),
+    make_spec<M_32x8_r8>("f32_m32x8_r8", 0.782, 1.0),
+    make_spec<M_8x8_l4r4>("f32_m8x8_l4r4", 0.750, 1.0),
+    make_spec<M_16x16_r4>("f32_m16x16_r4", 0.677, 1.0),
+    make_spec<M_16x16_r8>("f32_m16x16_r8", 0.703, 1.0),
+    make_spec<M_8x8_l4r8>("f32_m8x8_l4r8", 0.745, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f32(int *count) {

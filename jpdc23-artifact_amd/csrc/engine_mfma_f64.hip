@@ -17,10 +17,10 @@ using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
 using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4>;
 
 static const EngineSpec specs[] = {
-    make_spec<D_32x32>("f64_m32x32", 0.75, 1.0),
-    make_spec<D_32x16>("f64_m32x16", 0.80, 1.0),
-    make_spec<D_32x8_r4>("f64_m32x8_r4", 0.78, 1.0),
-    make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.90, 1.0),
+    make_spec<D_32x32>("f64_m32x32", 0.696, 1.0),
+    make_spec<D_32x16>("f64_m32x16", 0.697, 1.0),
+    make_spec<D_32x8_r4>("f64_m32x8_r4", 0.705, 1.0),
+    make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.730, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f64(int *count) {

@@ -27,12 +27,15 @@ struct EngineSpec {
     int threads;
     // launches the kernel; `args` points at an EngineArgs<T> of the matching type
     hipError_t (*launch)(const void *args, unsigned grid, hipStream_t stream);
-    // workgroups of this kernel that one CU holds at a time (registers and LDS), asked of the runtime once
-    int (*resident_blocks)();
+    // workgroups of this kernel that one CU of the current device holds at a time (registers and LDS), asked of the runtime
+    // once per device; 0 without a device
+    int (*resident_blocks_of_device)();
     // calibration of the planner's run-time model for grouped tiles: FMA issue slots a wavefront spends per
     // useful FMA instruction (LDS reads, waits and address arithmetic included), and the relative cost
     // of staging one band
     double issue_factor, stage_factor;
+    // the same, with the figure of an MI355X where no device can be asked (planning without a GPU)
+    int resident_blocks() const;
     int TXW() const { return LX * B; }
     int TYW() const { return LY * A; }
     int TXB() const { return TXW() * WX; }
@@ -92,7 +95,7 @@ int resident_blocks_engine() {
         if (allow_large_lds<C>() != hipSuccess ||
             hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, exp_lds<C>()) != hipSuccess || n < 1) {
             (void)hipGetLastError();
-            n = 1;
+            return 0; // (not kept: a device may appear later)
         }
         blocks[dev] = n;
     }

@@ -139,7 +139,7 @@ def test_tiles_with_copies_of_the_x_shifts(oracle):
         assert np.array_equal(xc.run("multimat_both_grouped", left, right, 45, n_left=3, n_right=15, params=xc.make_params(specialisation=index, rows_per_thread=16)), exp)
     left, right = rng.standard_normal((1, 128, 128)).astype(np.float32), rng.standard_normal((64, 128, 128)).astype(np.float32)
     got = xc.run("multimat_right_grouped", left, right, 64, n_left=1, n_right=64)
-    # assert "_m16x16_r4" in xc.last_launch()["kernel"], xc.last_launch()["kernel"]  # TODO(planner re-tune)
+    assert "_m16x16_r4" in xc.last_launch()["kernel"], xc.last_launch()["kernel"]
     sample = [0, 17, 63]
     assert rel_frob(got[sample], oracle.one_to_many(left, right[sample], threads=4)) <= 1e-5
 
