@@ -443,8 +443,10 @@ def main():
             (result if name == "C2" else per[name])["vector_fma_tiles"] = {k: entry[k] for k in ("kernel", "kernel_ms", "achieved", "frac", "bound", "steps")}
         # C2 launched two more ways: every accumulator running over its whole overlap like a thread of the reference's kernels
         # (xcorr_shuffle, distribution_type none: the launch that meets the 1e-5 bar against the fp32 host loop), and the
-        # grouped launch without atomic adds (whole reductions per work item: the same bits every run).
-        variants = {"C2_strict": ("shuffle", '{"distribution_type": 1}', 3), "C2_no_atomics": ("grouped_overlap", '{"rows_per_thread": 1024, "column_chunks": 1}', 5)}
+        # grouped launch without atomic adds (whole reductions per work item: the same bits every run), and the split launch
+        # whose chunks add themselves in order (xcorr_grouped_overlap_ordered_f32: no atomics, the same bits every run, no allocation).
+        variants = {"C2_strict": ("shuffle", '{"distribution_type": 1}', 3), "C2_no_atomics": ("grouped_overlap", '{"rows_per_thread": 1024, "column_chunks": 1}', 5),
+                    "C2_ordered": ("grouped_overlap_ordered", "{}", 5)}
         for key, (family, params_json, steps) in variants.items():
             v, entry = timed_variant(xc, workloads, "C2", family, params_json, steps, 1)
             if oracle is not None:

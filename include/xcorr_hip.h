@@ -293,6 +293,26 @@ int xcorr_grouped_overlap_f32(const float *left, const float *right, float *out,
 int xcorr_grouped_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                               const xcorr_params *p, void *stream);
 
+/* The same launcher with the chunks of a split reduction added IN ORDER instead of atomically. No counterpart in the
+ * reference; for callers that can neither allocate nor tolerate run-to-run differences: code under HIP graph capture,
+ * serving loops, harnesses that compare bits. Arguments and results as xcorr_grouped_overlap_f32 (same tiles, same
+ * choice of chunk; `out` need not be zeroed and is not cleared), but
+ *   - the launch never uses atomic adds (xcorr_last_launch().uses_atomics == 0): chunk 0 of a result tile stores, every
+ *     later chunk waits for its predecessor's ticket and adds itself on top, so every output is summed in the same order
+ *     every run: the same bits every run, at the speed of the split launch (a pair of 1024 x 1024: about 1 % slower);
+ *   - the tickets (32 bits per result tile of the launch) live in a fixed 4 MiB array inside the library's code object,
+ *     one copy per device, held until the process ends. The entry point allocates nothing and frees nothing. Launches
+ *     whose tiles outnumber the array (1 048 576: beyond any single pair of 16384 x 16384) return XCORR_ERR_UNSUPPORTED;
+ *   - all calls on one device share that array, which is cleared (by a kernel on `stream`) at the start of every call:
+ *     calls of this entry point that overlap in time on one device - different streams, different host threads - race
+ *     and give wrong results; calls on one stream, or otherwise ordered one after the other, are safe;
+ *   - `out` must be ordinary device memory that every compute unit reads and writes coherently through memory
+ *     (hipMalloc); only the matrix-core tiles run this way (matrix_cores = 2 is refused, column_chunks must be 0 or 1).
+ * A small pair that the launcher serves with the whole-pair-in-LDS kernel, and launches that do not split, run exactly as
+ * under xcorr_grouped_overlap_f32 (they never used atomics). */
+int xcorr_grouped_overlap_ordered_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                      const xcorr_params *p, void *stream);
+
 /* Multi-matrix-right: one left matrix against n_right right matrices, each lane
  * reuses a left value for p->right_matrices_per_thread right matrices.
  * Replaces run_ccn_shuffle_multimat_right_work_distribution<DIST> (kernels.cuh:130-142;

@@ -281,6 +281,7 @@ FAMILIES = {
     "shuffle": ("xcorr_shuffle", "pair", False),
     "split_row": ("xcorr_split_row", "pair", True),
     "grouped_overlap": ("xcorr_grouped_overlap", "pair", False),
+    "grouped_overlap_ordered": ("xcorr_grouped_overlap_ordered", "pair", False),  # fp32 only
     "multimat_right": ("xcorr_multimat_right", "right", None),
     "multimat_right_groups": ("xcorr_multimat_right_groups", "both", None),
     "multimat_right_grouped": ("xcorr_multimat_right_grouped", "both", False),

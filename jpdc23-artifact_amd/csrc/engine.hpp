@@ -42,7 +42,7 @@ struct EngineArgs {
     int nV, nU;         // matrix counts
     int group_m;        // 0: all pairs, out index v*nU + u. >0: left v pairs with right [v*m, (v+1)*m), out index = right index
     int rows_per_chunk; // left rows one work item reduces over
-    int dist;           // 0 none, 1 rectangle, 2 triangle (how worker ids map to (y tile, chunk))
+    int dist;           // 0 none, 1 rectangle, 2 triangle, 3 triangle by levels (how worker ids map to (y tile, chunk))
     int atomic;         // 1: atomicAdd partial sums into a zeroed output
     int ntx, nty;       // number of block tiles in x and y
     int nworkers_y;     // number of (y tile, chunk) workers
@@ -58,6 +58,11 @@ struct EngineArgs {
     // last block of a queue zeroes its pair again.
     // nullptr: block b takes the items b, b + gridDim.x, ... (with one block per work item: exactly one).
     int queues;
+    // Ordered accumulation (matrix-core sweep, dist 3): tickets[tile] is the chunk of the tile that may add itself to the output
+    // next. Chunk 0 stores, chunk c waits for tickets[tile] == c, adds itself to what is there and passes the ticket on; the last
+    // chunk leaves 0. The sums of a tile are thus always formed in chunk order: the same bits every run, no atomic adds, no
+    // cleared output. All zero before the launch. nullptr: off.
+    unsigned *tickets;
     unsigned *queue;
 };
 
@@ -169,6 +174,7 @@ __device__ __host__ __forceinline__ void tile_rows(int ty, int H, int &lo, int &
 // What one workgroup works on: a block tile of shifts, a group of matrices, a chunk of left rows and (when the columns
 // are cut) a chunk of right columns.
 struct WorkItem {
+    int tile, chunk, chunks;       // which tile of the launch (matrix group, x tile, y tile), which chunk of its rows, of how many
     int clo, chi;                  // left rows [clo, chi)
     int syb, sxb;                  // first y / x shift of the block tile
     int v_first, u_first, u_limit; // first left matrix, first right matrix, end of the right matrices this left group meets
@@ -187,13 +193,13 @@ __device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, int ite
     const int mat = item % (g.nvg * g.nug);
     item /= (g.nvg * g.nug);
     const int rc = g.rows_per_chunk;
-    const int worker = item % g.nworkers_y;
-    const int txi = item / g.nworkers_y;
+    // (by levels: `item` numbers (level, x tile, y tile of the level), decoded below)
+    const int worker = g.dist == 3 ? item : item % g.nworkers_y;
+    int txi = g.dist == 3 ? 0 : item / g.nworkers_y;
     const int ug = mat % g.nug, vg = mat / g.nug;
     // x and y tiles are visited centre-out: the block index order is the dispatch order, and
     // central tiles have the longest overlaps, so the longest work items start first
     const int txc = g.ntx / 2, tyc = g.nty / 2;
-    const int tx = (txi & 1) ? txc - (txi + 1) / 2 : txc + txi / 2;
 
     int tyi, chunk;
     if (g.dist == 0) {
@@ -202,6 +208,28 @@ __device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, int ite
     } else if (g.dist == 1) {
         tyi = worker % g.nty;
         chunk = worker / g.nty;
+    } else if (g.dist == 3) {
+        // by levels: first chunk 0 of every tile of the launch (x tiles slowest, y tiles fastest, as in the other orders), then
+        // chunk 1 of the tiles that have one, ... - a tile's chunks lie a whole level of the launch apart in launch order, so
+        // that one has long finished when the next wants to add itself on top (ordered accumulation).
+        // The y tiles with more than R rows are those from R / TYB to (2H - 2 - R) / TYB.
+        int w = worker, R = 0;
+        chunk = 0;
+        tyi = -1;
+        for (; R < H; ++chunk, R += rc) {
+            const int lo = R / C::TYB;
+            int hi = (2 * H - 2 - R) / C::TYB;
+            if (hi > g.nty - 1) hi = g.nty - 1;
+            const int n = hi - lo + 1;
+            if (n <= 0) continue;
+            if (w < n * g.ntx) {
+                txi = w / n;
+                tyi = lo + w % n;
+                break;
+            }
+            w -= n * g.ntx;
+        }
+        if (tyi < 0) return false;
     } else {
         int w = worker;
         tyi = 0;
@@ -215,9 +243,14 @@ __device__ __forceinline__ bool decode_work_item(const EngineArgs<T> &g, int ite
         chunk = w;
         if (tyi >= g.nty) return false;
     }
-    const int ty = (tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2;
+    const int tx = (txi & 1) ? txc - (txi + 1) / 2 : txc + txi / 2;
+    // (by levels the y tiles are taken in ascending order: all chunks of a level are equally long)
+    const int ty = g.dist == 3 ? tyi : (tyi & 1) ? tyc - (tyi + 1) / 2 : tyc + tyi / 2;
     int row_lo, row_hi;
     tile_rows<C>(ty, H, row_lo, row_hi);
+    wi.tile = (mat * g.ntx + tx) * g.nty + ty;
+    wi.chunk = chunk;
+    wi.chunks = (row_hi - row_lo + rc - 1) / rc;
     wi.clo = row_lo + chunk * rc;
     wi.chi = wi.clo + rc;
     if (wi.chi > row_hi) wi.chi = row_hi;

@@ -150,6 +150,7 @@ static long count_chunks(const EngineSpec &s, int H, int nty, int rc, int *max_c
 static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int xc, EnginePlan &plan) {
     plan.spec = &s;
     plan.predicted_us = 0;
+    plan.ordered = false;
     plan.x_chunks = 1;
     plan.x_chunk_cols = rq.W;
     if (xc > 1 && (rq.may_split || rq.caller_zeroes)) {
@@ -181,6 +182,11 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
         dist = 0;
         plan.atomic = 1;
         plan.zero_fill = true;
+    } else if (rq.ordered && plan.x_chunks == 1) {
+        dist = 3;
+        plan.atomic = 0;
+        plan.zero_fill = false;
+        plan.ordered = true;
     } else {
         if (dist <= 0) dist = 2;
         plan.atomic = 1;
@@ -240,7 +246,7 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
                                     : lanes_over_matrices ? (f32 ? 4.5e-6 : 3.0e-6) : (f32 ? 1.6e-6 : 4.4e-6);
     const double cyc = (f32 ? 2.0 : 4.0) / 2100.0; // microseconds per FMA instruction of a wavefront
     const double W = rq.W, H = rq.H, TXW = s.TXB(), TYW = s.TYB();
-    const bool split = plan.atomic != 0;
+    const bool split = plan.atomic != 0 || plan.ordered;
     const double rc = plan.rows_per_chunk;
     // a tile overlaps cols_tile right columns on average; cut into chunks, ceil(cols_tile / chunk) of its
     // x_chunks work items find columns, the others return at once
@@ -282,7 +288,8 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
                 k_tail * (item_time(inst_max, stages_max, occ) - item_time(inst_avg, stages_avg, occ));
         }
     }
-    if (split) t += t_clear + items * 64.0 * s.NV * s.NU * s.A * s.B * us_per_atomic;
+    // (chunks that add themselves in order: a read and a write of the tile through to memory per item, as an atomic add is)
+    if (split) t += (plan.ordered ? 0.0 : t_clear) + items * 64.0 * s.NV * s.NU * s.A * s.B * us_per_atomic;
     // Sustained vector-FMA load pulls the power-managed shader clock from 2.35 to 2.0-2.1 GHz within the first milliseconds
     // of a launch (random operands); the matrix cores hold 2.35 GHz on the same data. Measured / predicted run time of the
     // register tiles is 1.0 below half a millisecond and 1.3 from five milliseconds on, of the matrix-core tiles 1.1
@@ -304,6 +311,7 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         const EngineSpec &s = specs[i];
         if (rq.spec_index > 0 ? i != (int)rq.spec_index - 1 : s.A == 1) continue;
         if (rq.group_m > 0 ? (s.NVB() != 1 && !s.PG) : s.PG != 0) continue; // lanes over left matrices: all pairs, or paired groups
+        if (rq.ordered && !s.MFMA) continue;
         if (rq.spec_index == 0) {
             if (rq.matrix_cores == 1 ? !s.MFMA : rq.matrix_cores == 2 ? s.MFMA != 0 : false) continue;
             // The tiles whose columns hold copies of the x shifts win up to about 256x256 matrices (2-7 % over their 32 x 8
@@ -490,6 +498,31 @@ int plan_engine(const EngineRequest &rq, EnginePlan &plan) {
     return shape_plan(*best, rq, rc, xc > 1 ? xc : 1, plan);
 }
 
+// ---- scratch of the launches that add the chunks of a split reduction in order ----
+// One ticket (32 bits) per result tile of the launch, in a fixed array that belongs to the library's code object: nothing is
+// allocated. Every device that runs the library holds its own copy until the process ends; its address there is asked of the
+// runtime once per device (the array's name is a host-side stand-in, not a device address). All launches on a device share the
+// array: ordered launches that overlap in time on one device race for it.
+constexpr size_t SCRATCH_WORDS = 1u << 20; // 4 MiB: a single pair of up to 16384 x 16384 elements in tiles of 32 x 32 shifts
+static __device__ __align__(256) unsigned scratch[SCRATCH_WORDS];
+
+static unsigned *scratch_of_device() {
+    static unsigned *address[MAX_DEVICES] = {};
+    static std::mutex lock;
+    std::lock_guard<std::mutex> guard(lock);
+    const int dev = current_device();
+    if (address[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        address[dev] = static_cast<unsigned *>(p);
+    }
+    return address[dev];
+}
+size_t ordered_scratch_tiles() { return SCRATCH_WORDS; }
+
 // ---- work queues of persistent launches ----
 // A persistent launch (matrix-core sweep, more work items than the device holds blocks) hands out its work items through a
 // counter in device memory. Launches on one stream run one after the other, so every stream gets a counter pair of its own, in
@@ -569,6 +602,17 @@ static int launch_typed(const EngineRequest &rq, const EnginePlan &plan, hipStre
     a.x_chunk_cols = plan.x_chunk_cols;
     a.queue = nullptr;
     a.queues = 1;
+    a.tickets = nullptr;
+    if (plan.ordered) {
+        const size_t tiles = (size_t)plan.nvg * plan.nug * plan.ntx * plan.nty;
+        unsigned *tickets = scratch_of_device();
+        if (tickets == nullptr) return fail(XCORR_ERR_RUNTIME, "%s: the library's scratch array is not reachable on this device", rq.family);
+        if (tiles > SCRATCH_WORDS) return fail(XCORR_ERR_UNSUPPORTED, "%s: %zu result tiles need more tickets than the scratch array holds (%zu)", rq.family, tiles, SCRATCH_WORDS);
+        // (a kernel, not a memset: the launch may be captured into a graph)
+        zero_fill_kernel<unsigned><<<dim3((unsigned)((tiles + 255) / 256)), dim3(256), 0, stream>>>(tickets, tiles);
+        XCORR_HIP(hipGetLastError());
+        a.tickets = tickets;
+    }
     if (plan.zero_fill) {
         size_t n = (size_t)(2 * rq.W - 1) * (2 * rq.H - 1) * (rq.group_m > 0 ? (size_t)rq.nU : (size_t)rq.nV * rq.nU);
         size_t blocks = (n + 256 * 8 - 1) / (256 * 8);
@@ -596,7 +640,7 @@ static bool same_shape(const EngineRequest &a, const EngineRequest &b) {
            a.group_m == b.group_m && a.y_shifts == b.y_shifts && a.x_shifts == b.x_shifts && a.left_mats == b.left_mats &&
            a.right_mats == b.right_mats && a.lanes_x == b.lanes_x && a.lanes_y == b.lanes_y && a.waves == b.waves &&
            a.spec_index == b.spec_index && a.rows_per_worker == b.rows_per_worker && a.column_chunks == b.column_chunks && a.matrix_cores == b.matrix_cores &&
-           a.dist == b.dist && a.caller_zeroes == b.caller_zeroes && a.may_split == b.may_split;
+           a.dist == b.dist && a.caller_zeroes == b.caller_zeroes && a.may_split == b.may_split && a.ordered == b.ordered;
 }
 
 static int cached_plan(const EngineRequest &rq, EnginePlan &plan) {
@@ -676,7 +720,7 @@ int run_engine(const EngineRequest &request, hipStream_t stream) {
     rec.waves_x = plan.spec->WX;
     rec.waves_y = plan.spec->WY;
     rec.rows_per_worker = plan.rows_per_chunk;
-    rec.distribution_type = plan.dist == 0 ? XCORR_DIST_NONE : plan.dist == 1 ? XCORR_DIST_RECTANGLE : XCORR_DIST_TRIANGLE;
+    rec.distribution_type = plan.dist == 0 ? XCORR_DIST_NONE : plan.dist == 1 ? XCORR_DIST_RECTANGLE : XCORR_DIST_TRIANGLE; // (3, by levels: triangle)
     rec.uses_atomics = plan.atomic;
     rec.blocks_per_cu = plan.spec->resident_blocks();
     rec.column_chunks = plan.x_chunks;

@@ -140,6 +140,8 @@ struct EngineRequest {
     unsigned dist;            // XCORR_DIST_*
     bool caller_zeroes;       // true: split-row contract, output arrives zeroed, always accumulate atomically
     bool may_split;           // planner may split the reduction and clear the output itself
+    bool ordered;             // a split reduction adds its chunks in order (tickets in the library's scratch array, matrix-core
+                              // tiles only): no atomic adds, no cleared output, the same bits every run
 };
 
 struct EnginePlan {
@@ -148,6 +150,7 @@ struct EnginePlan {
     int rows_per_chunk, dist, atomic, total_items;
     int x_chunks, x_chunk_cols; // chunks of right columns per tile (1: not cut) and their width
     bool zero_fill;
+    bool ordered; // chunks add themselves to the output in order (dist 3, tickets)
     unsigned grid;
     double predicted_us; // of the run-time model (grouped families; 0 where no model was asked)
 };

@@ -285,7 +285,7 @@ int split_row_impl(const T *left, const T *right, T *out, unsigned cols, unsigne
 
 template <typename T>
 int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
-                 void *stream) {
+                 void *stream, bool ordered = false) {
     const LoadedParams loaded(pp);
     if (loaded.error) return loaded.error;
     const xcorr_params &p = loaded.p;
@@ -307,10 +307,16 @@ int grouped_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     const bool small = pair_fits_lds<T>(cols, rows) && cols <= 128 && elems <= (sizeof(T) == 4 ? 96u * 96u : 64u * 64u);
     if (p.whole_pair_in_lds == 1 || (p.whole_pair_in_lds == 0 && !tile_asked && small))
         return run_pair_in_lds<T>("grouped_overlap", left, right, out, cols, rows, as_stream(stream));
-    EngineRequest rq = base_request("grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);
+    EngineRequest rq = base_request(ordered ? "grouped_overlap_ordered" : "grouped_overlap", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = p.shifts_per_thread == 1 ? 2 : p.shifts_per_thread; // 0 = planner's choice among the grouped tiles
     rq.rows_per_worker = p.rows_per_thread;
     rq.may_split = true;
+    rq.ordered = ordered;
+    if (ordered) {
+        if (p.column_chunks > 1) return fail(XCORR_ERR_INVALID_ARGUMENT, "grouped_overlap_ordered: the columns of a reduction are not cut (column_chunks %u)", p.column_chunks);
+        if (p.matrix_cores == 2) return fail(XCORR_ERR_UNSUPPORTED, "grouped_overlap_ordered: only the matrix-core tiles add their chunks in order");
+        rq.column_chunks = 1;
+    }
     return run_engine(rq, as_stream(stream));
 }
 
@@ -488,6 +494,11 @@ int xcorr_block_per_overlap_f64(const double *left, const double *right, double 
 XCORR_PAIR_ENTRY(xcorr_shuffle, shuffle_impl)
 XCORR_PAIR_ENTRY(xcorr_split_row, split_row_impl)
 XCORR_PAIR_ENTRY(xcorr_grouped_overlap, grouped_impl)
+
+int xcorr_grouped_overlap_ordered_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
+                                      const xcorr_params *p, void *stream) {
+    return grouped_impl<float>(left, right, out, cols, rows, p, stream, true);
+}
 
 int xcorr_multimat_right_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                              unsigned n_right, const xcorr_params *p, void *stream) {
