@@ -111,15 +111,15 @@ typedef struct xcorr_params {
     /* warp-per-overlap through LDS (one_to_one.hpp:568-572) and block-per-overlap (one_to_one.hpp:649) */
     unsigned shared_mem_row_size;            /* columns staged per pass; this build always stages 64 (one per lane) */
     unsigned shared_mem_rows;                /* right rows staged per pass; 0 = shifts_per_thread_block, smaller is an error */
-    unsigned right_matrices_per_block;       /* 0 = 1; <= 8 */
+    unsigned right_matrices_per_block;       /* 0 = 8 (never more than there are); <= 8 */
     unsigned strided_load;                   /* load pattern of the reference's staging; no effect here */
     unsigned column_group_per_block;         /* 1: one block per group of 64 columns, sums added atomically (caller zeroes `out`) */
     unsigned block_size;                     /* block-per-overlap: threads per block, 0 = 128, <= 1024 */
     unsigned column_chunks;                  /* engine families: cut the reduction over right columns into this many chunks
                                                 (atomic adds, like rows_per_thread for rows); 0 = planner decides, no counterpart in the reference */
-    unsigned whole_pair_in_lds;              /* grouped-overlap, one small pair: 0 = the launcher decides, 1 = always run the kernel that
-                                                keeps both matrices in LDS (an error if they do not fit), 2 = never; no counterpart
-                                                in the reference */
+    unsigned whole_pair_in_lds;              /* few small matrices (see "Few small matrices" below): 0 = the launcher decides, 1 = always
+                                                run the kernel that keeps both matrices of a pair in LDS (an error if they do not
+                                                fit), 2 = never; no counterpart in the reference */
     unsigned matrix_cores;                   /* engine families: 0 = the launcher decides between its register tiles (vector FMA) and
                                                 its matrix-core tiles (v_mfma), 1 = matrix-core tiles only, 2 = never; the one-output-row
                                                 launchers (shuffle, split_row, multimat_right, multimat_both) take a matrix-core tile
@@ -174,7 +174,7 @@ const char *xcorr_version(void);
  * geometry, fill the launch record and return without launching or reading the pointers. Works without a GPU (256
  * CUs and the occupancies of an MI355X are assumed then); for tools and tests that ask what a call would run.
  * on = 2 plans as if `out` were memory the floating-point atomic add is not defined on (host-mapped, managed): a launch
- * that would split by the launcher's own choice stays whole, one whose contract is atomic adds is refused. */
+ * that names no chunk stays whole (plain stores), one whose chunk the caller fixed is refused. */
 int xcorr_plan_only(int on);
 
 /* ---- memory / queue shims: the C++ host never includes the HIP headers.
@@ -263,6 +263,18 @@ int xcorr_block_per_overlap_f32(const float *left, const float *right, float *ou
 int xcorr_block_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                 const xcorr_params *p, void *stream);
 
+/* Few small matrices. A launch is short of work for 256 CUs when its matrices are few and small, and what it costs then is
+ * the number of kernels it takes and the latency of one block. xcorr_shuffle, xcorr_split_row, xcorr_multimat_right(_groups),
+ * xcorr_multimat_both, xcorr_grouped_overlap, the work-distribution variant of xcorr_warp_per_overlap and
+ * xcorr_warp_per_overlap_lds therefore hand such a launch to one kernel of another kind when the call names no tile, no
+ * chunk of rows or columns and none of the LDS family's staging sizes: every block keeps both matrices of ITS pair whole in
+ * LDS and its wavefronts reduce groups of four adjacent x shifts over all rows (the role of run_ccn_warp_per_shift_shared_mem,
+ * kernels.cuh:144-161, at such sizes). One launch, plain stores, the same bits every run: `out` need not be zeroed whatever
+ * the family's contract says (xcorr_last_launch().uses_atomics == 0; a caller that plans first - xcorr_plan_only - may skip
+ * its clear, the `cross` binary does). Taken for one pair up to 96 x 96 fp32 / 64 x 64 fp64, and for at most 64 pairs of up to
+ * 32 x 32 with at most 2^24 multiply-adds in all; p->whole_pair_in_lds = 1 forces it (any number of pairs that fit), 2 keeps the
+ * family's own kernels. */
+
 /* Sliding-window base: every lane owns adjacent x shifts of one output row.
  * Replaces run_ccn_shuffle (kernels.cuh:65-73). One pair. Uses p->warps_per_thread_block. */
 int xcorr_shuffle_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
@@ -273,7 +285,8 @@ int xcorr_shuffle_f64(const double *left, const double *right, double *out, unsi
 /* Split-row: the overlap rows of an output row are split over several workers of at
  * most p->rows_per_thread rows each, partial sums are added atomically.
  * Replaces run_ccn_shuffle_work_distribution<DIST> (kernels.cuh:75-85). One pair.
- * THE CALLER ZEROES `out` FIRST (reference one_to_one.hpp:276-277). */
+ * THE CALLER ZEROES `out` FIRST (reference one_to_one.hpp:276-277). A launch that ends up with one work item per result tile
+ * (rows left whole, columns not cut) stores instead of adding: xcorr_last_launch().uses_atomics tells, also from a planning call. */
 int xcorr_split_row_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                         const xcorr_params *p, void *stream);
 int xcorr_split_row_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
@@ -282,12 +295,8 @@ int xcorr_split_row_f64(const double *left, const double *right, double *out, un
 /* Grouped-overlap: every lane accumulates p->shifts_per_thread adjacent y shifts.
  * Replaces run_ccn_shuffle_multirow_both (kernels.cuh:185-195). One pair.
  * `out` need not be zeroed: when the launcher splits the reduction to fill the
- * device it clears `out` itself on `stream` first. A pair small enough for both
- * matrices to sit in the LDS of one CU (run by default up to 96 x 96 fp32, 64 x 64 fp64) and given no tile
- * selection runs a kernel of its own kind instead: every block keeps the whole pair
- * in LDS and its wavefronts reduce groups of four adjacent x shifts, one launch,
- * no atomics (the role of run_ccn_warp_per_shift_shared_mem, kernels.cuh:144-161, at
- * such sizes); p->whole_pair_in_lds forces or forbids it. */
+ * device it clears `out` itself on `stream` first. A small pair given no tile
+ * selection runs whole in LDS ("Few small matrices" above). */
 int xcorr_grouped_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                               const xcorr_params *p, void *stream);
 int xcorr_grouped_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,

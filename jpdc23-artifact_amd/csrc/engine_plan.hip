@@ -172,6 +172,12 @@ static int shape_plan(const EngineSpec &s, const EngineRequest &rq, int rc, int 
         if (dist == 0) rc = rq.H;
         plan.atomic = 1;
         plan.zero_fill = false;
+        if (rc >= rq.H && plan.x_chunks == 1) {
+            // one work item per result tile: plain stores leave in a zeroed output what the atomic adds would (and need no
+            // zeroed output: a caller that looks at the record of a planning call first may skip its clear)
+            dist = 0;
+            plan.atomic = 0;
+        }
     } else if ((rc <= 0 || rc >= rq.H || !rq.may_split) && plan.x_chunks == 1) {
         rc = rq.H;
         dist = 0;
@@ -688,12 +694,15 @@ int run_engine(const EngineRequest &request, hipStream_t stream) {
     int rc = cached_plan(rq, plan);
     if (rc != XCORR_OK) return rc;
     if (plan.atomic && !atomics_defined_on(rq.out)) {
-        if (rq.caller_zeroes || !rq.may_split || rq.rows_per_worker != 0 || rq.column_chunks > 1)
+        if (rq.rows_per_worker != 0 || rq.column_chunks > 1)
             return fail(XCORR_ERR_UNSUPPORTED,
                         "%s: this launch adds partial sums with floating-point atomics, which are only defined on ordinary device memory "
                         "(hipMalloc); `out` is host-mapped, managed or unknown memory", rq.family);
-        // the launcher's own choice to split: the whole reduction per work item instead, plain stores
-        rq.may_split = false;
+        // no chunk named, the split is the launcher's own choice: the whole reduction per work item instead, plain stores
+        if (rq.caller_zeroes)
+            rq.dist = XCORR_DIST_NONE;
+        else
+            rq.may_split = false;
         rq.column_chunks = 1;
         if ((rc = cached_plan(rq, plan)) != XCORR_OK) return rc;
     }

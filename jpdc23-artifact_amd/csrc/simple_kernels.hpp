@@ -58,26 +58,45 @@ __device__ __forceinline__ void atomic_add_simple(double *p, double v) { unsafeA
 // eight element pairs are loaded ahead of the eight dependent FMAs so that the loads overlap.
 // ALL_PAIRS: every right matrix is correlated with every left matrix, result index = left * batch + right; the strip
 // holds `strip_lefts` result matrices and blockIdx.z walks (group of strip_lefts left matrices, right matrix).
-template <typename T, bool ALL_PAIRS>
+// STAGE (one left matrix, small matrices): the block first copies the left matrix and, per right matrix, that matrix into
+// LDS and the threads read their elements from there - same products, same order, less latency per load (the kernel is one
+// dependent chain of loads and FMAs per thread; a 24x24 pair: 22.0 -> 18.1 us, and 16.2 us with the last products of a row
+// loaded together instead of one by one; 16x16: 13.8 -> 8.9 us).
+template <typename T, bool ALL_PAIRS, bool STAGE>
 __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__ left, const T *__restrict__ right,
                                                             T *__restrict__ out, int W, int H, int n_left, int batch, int strip_lefts) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char overlap_smem[];
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
     const int strip_x = blockIdx.x * blockDim.x + threadIdx.x;
     const int oy = blockIdx.y * blockDim.y + threadIdx.y;
     const int in_strip = strip_x / Sx;
-    if (in_strip >= strip_lefts || oy >= Sy) return;
+    const bool active = in_strip < strip_lefts && oy < Sy;
+    if (!STAGE && !active) return;
     const int ox = strip_x - in_strip * Sx;
     const int sx = ox - (W - 1), sy = oy - (H - 1);
     const int xl_lo = sx > 0 ? sx : 0, xl_hi = W + sx < W ? W + sx : W;
     const int yl_lo = sy > 0 ? sy : 0, yl_hi = H + sy < H ? H + sy : H;
     const size_t in_area = (size_t)W * H, out_area = (size_t)Sx * Sy;
     const int steps = ALL_PAIRS ? (n_left / strip_lefts) * batch : batch;
+    const int tid = threadIdx.y * blockDim.x + threadIdx.x, nthreads = blockDim.x * blockDim.y;
+    T *Ls = reinterpret_cast<T *>(overlap_smem), *Rs = Ls + in_area;
+    if (STAGE)
+        for (int i = tid; i < (int)in_area; i += nthreads) Ls[i] = left[i];
     for (int z = blockIdx.z; z < steps; z += gridDim.z) {
         const int b = ALL_PAIRS ? z % batch : z;
         const int region = ALL_PAIRS ? (z / batch) * strip_lefts + in_strip : in_strip;
         const size_t mat = ALL_PAIRS ? (size_t)region * batch + b : (size_t)b * n_left + region;
         const T *l = left + region * in_area;
         const T *r = right + (ALL_PAIRS ? (size_t)b : mat) * in_area;
+        if (STAGE) { // (n_left == 1: region 0, right matrix b for every thread of the block)
+            __syncthreads(); // the previous right matrix is no longer read
+            const T *rz = right + (size_t)b * in_area;
+            for (int i = tid; i < (int)in_area; i += nthreads) Rs[i] = rz[i];
+            __syncthreads();
+            if (!active) continue;
+            l = Ls;
+            r = Rs;
+        }
         T sum = T(0);
         for (int yl = yl_lo; yl < yl_hi; ++yl) {
             const T *lrow = l + (size_t)yl * W;
@@ -93,7 +112,18 @@ __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__
 #pragma unroll
                 for (int i = 0; i < 8; ++i) sum += a[i] * c[i];
             }
-            for (; xl < xl_hi; ++xl) sum += rrow[xl] * lrow[xl];
+            if (xl < xl_hi) { // the last one to seven products: loaded together like a whole group (from addresses inside the row), added in order
+                T a[8], c[8];
+#pragma unroll
+                for (int i = 0; i < 7; ++i) {
+                    const int x = xl + i < xl_hi ? xl + i : xl;
+                    a[i] = rrow[x];
+                    c[i] = lrow[x];
+                }
+#pragma unroll
+                for (int i = 0; i < 7; ++i)
+                    if (xl + i < xl_hi) sum += a[i] * c[i];
+            }
         }
         out[mat * out_area + (size_t)oy * Sx + ox] = sum;
     }
@@ -119,10 +149,15 @@ int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsig
         if ((unsigned long long)n_left * batch > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: %u left, %u right", n_left, batch);
     }
     dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y, (unsigned)(steps < 65535 ? steps : 65535));
-    if (all_pairs)
-        overlap_wise_kernel<T, true><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
+    // one left matrix and a pair fits 64 KB of LDS: staged (the loops over right matrices per block stay short: gridDim.z covers them)
+    const size_t pair_bytes = 2 * (size_t)cols * rows * sizeof(T);
+    const bool stage = n_left == 1 && pair_bytes <= 64 * 1024;
+    if (stage)
+        overlap_wise_kernel<T, false, true><<<grid, block, pair_bytes, stream>>>(left, right, out, (int)cols, (int)rows, 1, (int)batch, 1);
+    else if (all_pairs)
+        overlap_wise_kernel<T, true, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
     else
-        overlap_wise_kernel<T, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
+        overlap_wise_kernel<T, false, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
     XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
@@ -328,7 +363,9 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
     }
     dim3 grid((Sx + spb - 1) / spb, grid_y);
     const int W = (int)cols, H = (int)rows;
-    if (variant == 0)
+    if (plan_only())
+        ; // (planning only: the record below is what a launch would report)
+    else if (variant == 0)
         warp_per_overlap_kernel<T, 0, 0><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
     else if (variant == 1)
         warp_per_overlap_kernel<T, 1, 0><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
@@ -338,7 +375,7 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
         warp_per_overlap_kernel<T, 2, 1><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
     else
         warp_per_overlap_kernel<T, 2, 2><<<grid, block, 0, stream>>>(left, right, out, W, H, max_rows);
-    XCORR_HIP(hipGetLastError());
+    if (!plan_only()) XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
     snprintf(rec.kernel, sizeof(rec.kernel), "warp_per_overlap/%s_v%d", sizeof(T) == 4 ? "f32" : "f64", variant);
@@ -372,6 +409,9 @@ int run_warp_per_overlap(const T *left, const T *right, T *out, unsigned cols, u
 struct PairGeometry {
     int W, H, pitch_l, pitch_r, tasks_x, total_tasks;
     unsigned magic_pl, magic_pr, magic_tx; // floor(2^32 / d) + 1 for d = pieces per left row, per right row, tasks per output row
+    // several pairs in one launch: blocks_per_pair consecutive blocks share a pair; pair p is left matrix p / left_div with right
+    // matrix p % right_mod (right_mod 0: right matrix p) and writes result p
+    int blocks_per_pair, left_div, right_mod;
 };
 __device__ __forceinline__ int div_by(int n, int d, unsigned magic) { return d == 1 ? n : (int)__umulhi((unsigned)n, magic); }
 
@@ -379,9 +419,13 @@ __device__ __forceinline__ int div_by(int n, int d, unsigned magic) { return d =
 // constants and every LDS read of a round is the round's base address plus an immediate offset (with run-time pitches
 // one address addition per read, two thirds as many instructions again as the FMAs).
 template <typename T, int A, int B, int U, int COLS>
-__global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left, const T *__restrict__ right, T *__restrict__ out,
+__global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left_all, const T *__restrict__ right_all, T *__restrict__ out_all,
                                                            const PairGeometry geo) {
     const int W = COLS ? COLS : geo.W, H = geo.H, tasks_x = geo.tasks_x, total_tasks = geo.total_tasks;
+    const int pair = (int)blockIdx.x / geo.blocks_per_pair, block_of_pair = (int)blockIdx.x % geo.blocks_per_pair;
+    const T *left = left_all + (size_t)(pair / geo.left_div) * W * H;
+    const T *right = right_all + (size_t)(geo.right_mod ? pair % geo.right_mod : pair) * W * H;
+    T *out = out_all + (size_t)pair * (2 * W - 1) * (2 * H - 1);
     const int pitch_l = COLS ? COLS + 2 * (B < 16 / (int)sizeof(T) ? 16 / (int)sizeof(T) : B) : geo.pitch_l, pitch_r = COLS ? COLS : geo.pitch_r;
     using vec = typename vec128<T>::type;
     constexpr int VK = 16 / (int)sizeof(T);
@@ -429,8 +473,8 @@ __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__
     __syncthreads();
     const int lane = tid & 63, wave = tid >> 6, nw = nt >> 6;
     const int Sx = 2 * W - 1, Sy = 2 * H - 1;
-    // task (wave w of block b, round i) = w * gridDim + b + i * gridDim * nw
-    for (int t = wave * (int)gridDim.x + (int)blockIdx.x; t < total_tasks; t += (int)gridDim.x * nw) {
+    // task (wave w of block b of the pair's blocks, round i) = w * blocks + b + i * blocks * nw
+    for (int t = wave * geo.blocks_per_pair + block_of_pair; t < total_tasks; t += geo.blocks_per_pair * nw) {
         const int ty = div_by(t, tasks_x, geo.magic_tx);
         const int oy0 = ty * A, ox0 = (t - ty * tasks_x) * B;
         const int sy0 = oy0 - (H - 1), sx0 = ox0 - (W - 1);
@@ -510,8 +554,13 @@ inline bool pair_fits_lds(unsigned cols, unsigned rows) {
     return pair_in_lds_bytes<T>(cols, rows, 2, 4) <= 160 * 1024;
 }
 
+// What the pairs of a launch are: n_pairs results; pair p = left p / left_div x right p % right_mod (0: right p).
+struct PairList {
+    unsigned n_pairs = 1, left_div = 1, right_mod = 0;
+};
+
 template <typename T, int A, int U, int COLS>
-int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, unsigned rows, size_t bytes, unsigned *grid_out,
+int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, unsigned rows, size_t bytes, const PairList &pairs, unsigned *grid_out,
                        unsigned *waves_out, hipStream_t stream) {
     constexpr unsigned VK = 16 / sizeof(T), B = PAIR_B, PAD = B < VK ? VK : B;
     const int pitch_l = (int)((cols + 2 * PAD + VK - 1) / VK * VK), pitch_r = (int)((cols + VK - 1) / VK * VK);
@@ -527,12 +576,17 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
     const unsigned tasks_x = (Sx + B - 1) / B, total = tasks_x * ((Sy + A - 1) / A);
     const int cus = device_cus();
     // eight wavefronts per block while that still gives every task a wavefront of its own, else sixteen
-    const unsigned waves = total <= 8u * (unsigned)cus ? 8 : 16;
+    const unsigned waves = (size_t)total * pairs.n_pairs <= 8u * (size_t)cus ? 8 : 16;
     unsigned grid = (total + waves - 1) / waves;
-    if (grid > (unsigned)cus) grid = (unsigned)cus; // one block per CU: every block pays for its own copy of the pair
+    // one block per CU: every block pays for its own copy of the pair (several pairs: the CUs are dealt to them, two blocks
+    // per CU where two fit)
+    const unsigned slots = (unsigned)cus * (pairs.n_pairs > 1 && bytes <= 64 * 1024 ? 2u : 1u);
+    const unsigned share = slots / pairs.n_pairs > 0 ? slots / pairs.n_pairs : 1;
+    if (grid > share) grid = share;
     auto magic = [](unsigned d) { return (unsigned)((1ull << 32) / d) + 1u; }; // exact for n * d < 2^32, far above any index here
     const PairGeometry geo = {(int)cols,         (int)rows,          pitch_l,       pitch_r, (int)tasks_x, (int)total,
-                              magic(pitch_l / VK), magic(pitch_r / VK), magic(tasks_x)};
+                              magic(pitch_l / VK), magic(pitch_r / VK), magic(tasks_x), (int)grid, (int)pairs.left_div, (int)pairs.right_mod};
+    grid *= pairs.n_pairs;
     if (!plan_only()) {
         pair_in_lds_kernel<T, A, B, U, COLS><<<dim3(grid), dim3(64 * waves), bytes, stream>>>(left, right, out, geo);
         XCORR_HIP(hipGetLastError());
@@ -543,7 +597,8 @@ int launch_pair_in_lds(const T *left, const T *right, T *out, unsigned cols, uns
 }
 
 template <typename T>
-int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, unsigned cols, unsigned rows, hipStream_t stream) {
+int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, unsigned cols, unsigned rows, hipStream_t stream,
+                    const PairList &pairs = PairList()) {
     if (!pair_fits_lds<T>(cols, rows)) return fail(XCORR_ERR_UNSUPPORTED, "%s: a %u x %u pair does not fit the LDS of a CU", family, rows, cols);
     // One y shift per task while the tasks are few (at 64x64 fp32 every wavefront slot of the device gets one task: the
     // kernel is bound by the latency of a task, not by LDS throughput), two beyond. Measured, microseconds per launch with
@@ -556,19 +611,19 @@ int run_pair_in_lds(const char *family, const T *left, const T *right, T *out, u
     int rc;
     // the column counts the reference's benchmarks use are compiled in (multiples of 16 whose pitches need no rounding)
     if (A == 1 && cols == 64)
-        rc = launch_pair_in_lds<T, 1, U, 64>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 1, U, 64>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else if (A == 1 && cols == 32)
-        rc = launch_pair_in_lds<T, 1, U, 32>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 1, U, 32>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else if (A == 1 && cols == 16)
-        rc = launch_pair_in_lds<T, 1, U, 16>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 1, U, 16>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else if (A == 1)
-        rc = launch_pair_in_lds<T, 1, U, 0>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 1, U, 0>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else if (cols == 64)
-        rc = launch_pair_in_lds<T, 2, U, 64>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 2, U, 64>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else if (cols == 96)
-        rc = launch_pair_in_lds<T, 2, U, 96>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 2, U, 96>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     else
-        rc = launch_pair_in_lds<T, 2, U, 0>(left, right, out, cols, rows, bytes, &grid, &waves, stream);
+        rc = launch_pair_in_lds<T, 2, U, 0>(left, right, out, cols, rows, bytes, pairs, &grid, &waves, stream);
     if (rc != XCORR_OK) return rc;
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
@@ -684,7 +739,7 @@ int run_warp_per_overlap_lds(const T *left, const T *right, T *out, unsigned col
     // reference limits: naive_warp_per_shift_shared_mem.cu:681-693
     if (p.shifts_per_thread_block > 32)
         return fail(XCORR_ERR_INVALID_ARGUMENT, "Too many shifts per block: %u (max 32)", p.shifts_per_thread_block);
-    unsigned nr = p.right_matrices_per_block ? p.right_matrices_per_block : 1;
+    unsigned nr = p.right_matrices_per_block ? p.right_matrices_per_block : 8; // (the reference's default, one_to_many.hpp:415)
     if (nr > 8) return fail(XCORR_ERR_INVALID_ARGUMENT, "Invalid number of right matrices per block: %u [1-8]", nr);
     if (nr > n_right) nr = n_right; // no bands and FMAs for matrices that do not exist
     unsigned nw = p.shifts_per_thread_block ? p.shifts_per_thread_block : 16;
@@ -703,7 +758,8 @@ int run_warp_per_overlap_lds(const T *left, const T *right, T *out, unsigned col
     const unsigned column_groups = p.column_group_per_block ? (cols + 63) / 64 : 1;
     dim3 block(64, nw), grid(Sx * groups, (Sy + nw - 1) / nw, column_groups);
     const int W = (int)cols, H = (int)rows;
-    switch (nr) {
+    switch (plan_only() ? 0u : nr) {
+    case 0: break; // (planning only: the record below is what a launch would report)
     case 1: launch_wpo_lds<T, 1>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
     case 2: launch_wpo_lds<T, 2>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
     case 3: launch_wpo_lds<T, 3>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
@@ -713,7 +769,7 @@ int run_warp_per_overlap_lds(const T *left, const T *right, T *out, unsigned col
     case 7: launch_wpo_lds<T, 7>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
     default: launch_wpo_lds<T, 8>(left, right, out, W, H, (int)n_right, (int)sr, grid, block, lds, stream); break;
     }
-    XCORR_HIP(hipGetLastError());
+    if (!plan_only()) XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
     snprintf(rec.kernel, sizeof(rec.kernel), "warp_per_overlap_lds/%s_r%u", sizeof(T) == 4 ? "f32" : "f64", nr);

@@ -245,6 +245,36 @@ EngineRequest base_request(const char *family, int elem_bytes, const void *left,
     return rq;
 }
 
+// Few small matrices and a call that names no tile or chunk: every pair whole in the LDS of its share of the
+// CUs (pair_in_lds_kernel), one launch, plain stores - whatever the family's contract says about a zeroed output (stores into
+// a zeroed output are what the atomic adds of one work item per tile would leave there). The launch record then says
+// uses_atomics = 0, and a caller that asks first (xcorr_plan_only) may skip its clear. Measured against the engine's launches
+// (with the clear kernel where the contract has one) through the `cross` binary, microseconds per launch: one pair up to
+// 96x96 fp32 / 64x64 fp64 as for xcorr_grouped_overlap; at most 64 pairs of up to 32x32 and 2^24 multiply-adds in all.
+// Whether a call of the sliding-window families names a tile or a chunk. (A distribution alone names neither: it says how a
+// split launch would cut the rows. With one pair the matrices per thread say nothing either.)
+bool names_tile_or_chunk(const xcorr_params &p, size_t n_pairs) {
+    return p.specialisation || p.x_shifts_per_thread || p.lanes_x || p.lanes_y || p.rows_per_thread || p.column_chunks || p.matrix_cores ||
+           p.shifts_per_thread || p.shifts_per_thread_right_matrix || p.shifts_per_thread_block ||
+           (n_pairs > 1 && (p.right_matrices_per_thread || p.left_matrices_per_thread));
+}
+
+template <typename T>
+bool small_pairs_in_lds(const xcorr_params &p, bool named, unsigned cols, unsigned rows, size_t n_pairs, int *error) {
+    *error = XCORR_OK;
+    if (p.whole_pair_in_lds > 2) {
+        *error = fail(XCORR_ERR_INVALID_ARGUMENT, "whole_pair_in_lds must be 0, 1 or 2, not %u", p.whole_pair_in_lds);
+        return false;
+    }
+    if (p.whole_pair_in_lds == 2) return false;
+    if (p.whole_pair_in_lds == 1) return true; // (an error from the launcher if the pair does not fit)
+    if (named || !pair_fits_lds<T>(cols, rows)) return false;
+    const size_t elems = (size_t)cols * rows;
+    if (n_pairs == 1) return cols <= 128 && elems <= (sizeof(T) == 4 ? 96u * 96u : 64u * 64u);
+    // (pairs of 32x32: 4.0 us for 2, 5.8 for 8, 8.8 for 16, 15.1 for 32 - where the engine's tiles take 9.4)
+    return cols <= 32 && rows <= 32 && n_pairs <= 64 && n_pairs * elems * elems <= (1u << 24);
+}
+
 template <typename T>
 int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp,
                  void *stream) {
@@ -254,6 +284,8 @@ int shuffle_impl(const T *left, const T *right, T *out, unsigned cols, unsigned 
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, 1), cols, rows, 1, &rc)) return run_pair_in_lds<T>("shuffle", left, right, out, cols, rows, as_stream(stream));
+    if (rc) return rc;
     EngineRequest rq = base_request("shuffle", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = 1;
     rq.left_mats = rq.right_mats = 1;
@@ -275,6 +307,8 @@ int split_row_impl(const T *left, const T *right, T *out, unsigned cols, unsigne
     if (rc) return rc;
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, 1), cols, rows, 1, &rc)) return run_pair_in_lds<T>("split_row", left, right, out, cols, rows, as_stream(stream));
+    if (rc) return rc;
     EngineRequest rq = base_request("split_row", sizeof(T), left, right, out, cols, rows, 1, 1, p);
     rq.y_shifts = 1;
     rq.left_mats = rq.right_mats = 1;
@@ -332,6 +366,13 @@ int multimat_right_impl(const T *left, const T *right, T *out, unsigned cols, un
     if ((rc = check_limit("warps per thread block", p.warps_per_thread_block, Limits::warps_per_block))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, (size_t)n_left * n_right), cols, rows, (size_t)n_left * n_right, &rc)) {
+        PairList pairs;
+        pairs.n_pairs = n_left * n_right;
+        pairs.left_div = n_right; // left l meets the right matrices [l * n_right, (l + 1) * n_right)
+        return run_pair_in_lds<T>("multimat_right", left, right, out, cols, rows, as_stream(stream), pairs);
+    }
+    if (rc) return rc;
     EngineRequest rq = base_request("multimat_right", sizeof(T), left, right, out, cols, rows, n_left, n_left * n_right, p);
     rq.group_m = n_left > 1 ? (int)n_right : 0; // left l against its own group of n_right right matrices
     rq.y_shifts = 1;
@@ -387,6 +428,14 @@ int multimat_both_impl(const T *left, const T *right, T *out, unsigned cols, uns
     if ((rc = check_limit("left matrices per thread", p.left_matrices_per_thread, Limits::left_matrices))) return rc;
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::right_matrices))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, (size_t)n_left * n_right), cols, rows, (size_t)n_left * n_right, &rc)) {
+        PairList pairs;
+        pairs.n_pairs = n_left * n_right;
+        pairs.left_div = n_right; // result l * n_right + r
+        pairs.right_mod = n_right;
+        return run_pair_in_lds<T>("multimat_both", left, right, out, cols, rows, as_stream(stream), pairs);
+    }
+    if (rc) return rc;
     EngineRequest rq = base_request("multimat_both", sizeof(T), left, right, out, cols, rows, n_left, n_right, p);
     rq.y_shifts = 1;
     rq.left_mats = p.left_matrices_per_thread;
@@ -421,6 +470,46 @@ int multimat_both_grouped_impl(const T *left, const T *right, T *out, unsigned c
     return run_engine(rq, as_stream(stream));
 }
 
+// The work-distribution variant (zeroed output, atomic adds of row chunks) on a small pair with no chunk named: the whole pair in LDS
+// instead, one launch, plain stores (small_pairs_in_lds); the other variants are the kernels their names say.
+template <typename T>
+int warp_per_overlap_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, const xcorr_params *pp, void *stream) {
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    if ((rc = check_limit("shifts per thread block", p.shifts_per_thread_block, 32))) return rc; // naive_warp_per_shift.cu:316-318
+    if ((rc = check_dist(p.distribution_type))) return rc;
+    if (p.warp_per_overlap_variant == XCORR_WPO_WORK_DISTRIBUTION) {
+        xcorr_params q = p;
+        q.shifts_per_thread_block = 0; // (the shape of a block, not a chunk of the work)
+        if (small_pairs_in_lds<T>(q, names_tile_or_chunk(q, 1), cols, rows, 1, &rc)) return run_pair_in_lds<T>("warp_per_overlap", left, right, out, cols, rows, as_stream(stream));
+        if (rc) return rc;
+    }
+    return run_warp_per_overlap<T>(left, right, out, cols, rows, p, as_stream(stream));
+}
+
+// The LDS-staged wavefront-per-overlap family on few small matrices with none of its staging parameters named: the kernel that
+// keeps every pair whole in LDS does the same work (a wavefront per group of overlaps, both matrices in LDS) in one pass.
+template <typename T>
+int warp_per_overlap_lds_impl(const T *left, const T *right, T *out, unsigned cols, unsigned rows, unsigned n_right, const xcorr_params *pp,
+                              void *stream) {
+    const LoadedParams loaded(pp);
+    if (loaded.error) return loaded.error;
+    const xcorr_params &p = loaded.p;
+    int rc = check_shape(left, right, out, cols, rows);
+    if (rc) return rc;
+    const bool named = p.shifts_per_thread_block || p.shared_mem_rows || p.shared_mem_row_size || p.right_matrices_per_block || p.column_group_per_block;
+    if (n_right > 0 && n_right <= 64 && small_pairs_in_lds<T>(p, named, cols, rows, n_right, &rc)) {
+        PairList pairs;
+        pairs.n_pairs = pairs.left_div = n_right;
+        return run_pair_in_lds<T>("warp_per_overlap_lds", left, right, out, cols, rows, as_stream(stream), pairs);
+    }
+    if (rc) return rc;
+    return run_warp_per_overlap_lds<T>(left, right, out, cols, rows, n_right, p, as_stream(stream));
+}
+
 } // namespace
 
 extern "C" {
@@ -444,28 +533,20 @@ int xcorr_overlap_wise_all_pairs_f64(const double *left, const double *right, do
 
 int xcorr_warp_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                                const xcorr_params *p, void *stream) {
-    const LoadedParams loaded(p);
-    if (loaded.error) return loaded.error;
-    return run_warp_per_overlap<float>(left, right, out, cols, rows, loaded.p, as_stream(stream));
+    return warp_per_overlap_impl<float>(left, right, out, cols, rows, p, stream);
 }
 int xcorr_warp_per_overlap_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                const xcorr_params *p, void *stream) {
-    const LoadedParams loaded(p);
-    if (loaded.error) return loaded.error;
-    return run_warp_per_overlap<double>(left, right, out, cols, rows, loaded.p, as_stream(stream));
+    return warp_per_overlap_impl<double>(left, right, out, cols, rows, p, stream);
 }
 
 int xcorr_warp_per_overlap_lds_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,
                                    unsigned n_right, const xcorr_params *p, void *stream) {
-    const LoadedParams loaded(p);
-    if (loaded.error) return loaded.error;
-    return run_warp_per_overlap_lds<float>(left, right, out, cols, rows, n_right, loaded.p, as_stream(stream));
+    return warp_per_overlap_lds_impl<float>(left, right, out, cols, rows, n_right, p, stream);
 }
 int xcorr_warp_per_overlap_lds_f64(const double *left, const double *right, double *out, unsigned cols, unsigned rows,
                                    unsigned n_right, const xcorr_params *p, void *stream) {
-    const LoadedParams loaded(p);
-    if (loaded.error) return loaded.error;
-    return run_warp_per_overlap_lds<double>(left, right, out, cols, rows, n_right, loaded.p, as_stream(stream));
+    return warp_per_overlap_lds_impl<double>(left, right, out, cols, rows, n_right, p, stream);
 }
 
 int xcorr_block_per_overlap_f32(const float *left, const float *right, float *out, unsigned cols, unsigned rows,

@@ -275,8 +275,11 @@ gpu_algorithm<T>::gpu_algorithm(const algorithm_def &def, const json_args &args,
         // (the split-row launchers of the sliding-window engine also take their chunk of rows from the library unless the file
         // names one: the reference's default of 10 rows leaves most of the GPU idle on small inputs and cuts large ones too short)
         const bool engine_split_row = def.family == Family::split_row || def.family == Family::multimat_right || def.family == Family::multimat_both;
+        // (and the staging parameters of the LDS wavefront-per-overlap family, whose defaults in the library are the reference's:
+        // with none of them named the library may keep few small matrices whole in LDS instead)
+        const bool lds_staging = def.family == Family::warp_per_overlap_lds && a.t == arg_spec::type::uint && a.field != nullptr;
         const bool library_default = !args.contains(a.key) && (selects_tile(a.key) || (engine_split_row && std::string(a.key) == "rows_per_thread") ||
-                                                               (def.family == Family::warp_per_overlap && std::string(a.key) == "rows_per_warp"));
+                                                               (def.family == Family::warp_per_overlap && std::string(a.key) == "rows_per_warp") || lds_staging);
         if (a.field) params_.*(a.field) = library_default ? 0u : value;
         if (a.report) props_.emplace_back(a.key, shown);
     }
@@ -390,12 +393,37 @@ void gpu_algorithm<T>::launch(const T *left, const T *right, T *out, dsize_t n_l
 
 template <typename T>
 void gpu_algorithm<T>::launch_all() {
+    // (the clear is a small fill kernel: shorter than a memset command for the outputs of small instances, and it may be captured)
+    if (clear_before_launch_) xcheck(xcorr_clear_async(d_results_, results_.size() * sizeof(T), nullptr));
+    launch_kernels();
+}
+
+// The families whose contract is a zeroed output are asked first what they would run on this instance (a planning call:
+// nothing is launched): a launch that adds nothing into the output - one work item per result tile, or a small instance
+// whose pairs run whole in LDS - stores every element, and the clear kernel in front of it would only cost time.
+template <typename T>
+bool gpu_algorithm<T>::launches_add_into_output() {
+    const bool plans = def_.family == Family::split_row || def_.family == Family::multimat_right || def_.family == Family::multimat_both ||
+                       def_.family == Family::warp_per_overlap || def_.family == Family::warp_per_overlap_lds;
+    if (!plans) return true;
+    xcorr_plan_only(1);
+    try {
+        launch_kernels();
+    } catch (...) {
+        xcorr_plan_only(0);
+        throw;
+    }
+    xcorr_plan_only(0);
+    xcorr_launch_record rec; // (the launches of one run all have the same shape: the last record speaks for them)
+    return xcorr_last_launch(&rec) != XCORR_OK || rec.uses_atomics != 0;
+}
+
+template <typename T>
+void gpu_algorithm<T>::launch_kernels() {
     const dsize_t n = refs_.num_matrices(), total_right = targets_.num_matrices();
     const std::size_t in_area = refs_.matrix_size().area(), out_area = results_.matrix_size().area();
-    // (the clear is a small fill kernel: shorter than a memset command for the outputs of small instances, and it may be captured)
-    if (zero_output_) xcheck(xcorr_clear_async(d_results_, results_.size() * sizeof(T), nullptr));
     if (def_.per_left_streams) {
-        if (zero_output_) xcheck(xcorr_device_sync()); // the clear runs on the default stream
+        if (clear_before_launch_) xcheck(xcorr_device_sync()); // the clear runs on the default stream
         // one launch per left matrix, left r on stream r mod k (n_to_mn.hpp:553-571, n_to_m.hpp:198-212)
         const bool all_pairs = def_.mode == Mode::n_to_m;
         const dsize_t per_left = all_pairs ? total_right : total_right / n;
@@ -419,6 +447,7 @@ void gpu_algorithm<T>::launch_all() {
 
 template <typename T>
 void gpu_algorithm<T>::run_impl() {
+    clear_before_launch_ = zero_output_ && launches_add_into_output();
     if (def_.per_left_streams) {
         // several streams: wall clock around launch + device synchronisation (n_to_mn.hpp:500-505)
         sw_.cpu_adaptive_measure(0, measure_alg(), true, [&] { launch_all(); });

@@ -252,8 +252,9 @@ protected:
 
 private:
     algorithm_def def_;
-    xcorr_params params_ = XCORR_PARAMS_INIT;
+    xcorr_params params_ = [] { xcorr_params p{}; p.struct_size = sizeof(xcorr_params); return p; }(); // (XCORR_PARAMS_INIT, without -Wextra's remarks)
     bool zero_output_ = false; // clear the output inside the measured block (split-row contract, column groups)
+    bool clear_before_launch_ = false; // ... and the launches of this instance do add into it
     properties props_;
     unsigned num_streams_ = 0;
     host_array refs_, targets_, results_;
@@ -261,6 +262,8 @@ private:
     std::vector<void *> streams_;
 
     void launch_all();
+    void launch_kernels();
+    bool launches_add_into_output();
     void report_effective_arguments();
     void release() noexcept;
     void launch(const T *left, const T *right, T *out, dsize_t n_left, dsize_t n_right, void *stream);

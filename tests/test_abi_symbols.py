@@ -169,7 +169,7 @@ def test_params_struct_size_rules():
 
 def test_split_plans_need_ordinary_device_memory():
     """Plan-only mode 2 plans for an output the float atomic add is not defined on (host-mapped, managed): the launcher's own
-    split is given up for the whole reduction per work item, a contract of atomic adds is refused."""
+    split is given up for the whole reduction per work item, a named chunk (which needs the atomic adds) is refused."""
     xc = load_package()
     lib = xc.lib()
     dummy = ctypes.c_void_p(16)
@@ -189,12 +189,21 @@ def test_split_plans_need_ordinary_device_memory():
     assert code == 0 and rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 512
     code, rec = ask("xcorr_shuffle_f32", 2, 64, 64, matrix_cores=2)
     assert code == 0 and rec["uses_atomics"] == 0
-    code, msg = ask("xcorr_split_row_f32", 2, 64, 64)
+    # a small pair runs whole in LDS whatever the memory; a large one of a zeroed-output family is replanned with whole rows
+    code, rec = ask("xcorr_split_row_f32", 2, 64, 64)
+    assert code == 0 and rec["uses_atomics"] == 0 and "pair_in_lds" in rec["kernel"]
+    code, rec = ask("xcorr_split_row_f32", 1, 512, 512)
+    assert code == 0 and rec["uses_atomics"] == 1
+    code, rec = ask("xcorr_split_row_f32", 2, 512, 512)
+    assert code == 0 and rec["uses_atomics"] == 0 and rec["rows_per_worker"] == 512 and rec["column_chunks"] == 1
+    code, msg = ask("xcorr_split_row_f32", 2, 512, 512, rows_per_thread=32)
     assert code == 3 and b"atomics" in msg
     code, msg = ask("xcorr_grouped_overlap_f32", 2, 512, 512, rows_per_thread=32)
     assert code == 3
-    code, rec = ask("xcorr_multimat_both_f64", 2, 32, 32, 4, 4)
+    code, rec = ask("xcorr_multimat_both_f64", 2, 64, 64, 4, 4, rows_per_thread=16)
     assert code == 3
+    code, rec = ask("xcorr_multimat_both_f64", 2, 64, 64, 4, 4)
+    assert code == 0 and rec["uses_atomics"] == 0
     assert lib.xcorr_plan_only(3) == 1
 
 

@@ -97,15 +97,25 @@ def test_json_arguments_and_properties(tmp_path, oracle):
     assert rc == 0, err
     header, row = (tmp_path / "t2.csv").read_text().strip().splitlines()
     assert header.endswith("warps_per_thread_block,rows_per_thread,distribution_type") and row.endswith("8,4,triangle")
-    # without rows_per_thread in the file the library picks the chunk (short ones for a single small pair, not the
-    # reference's 10) and the measurement file reports it
+    # without rows_per_thread in the file the library picks the chunk (not the reference's 10) and the measurement file
+    # reports it: a pair this small runs whole in LDS without any split (and the binary, which asks first, does not clear
+    # the output) ...
     args = write_args(tmp_path / "d.json", distribution_type="rectangle")
     rc, _, err = run_cross("run", "--args_path", args, "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / "t3.csv", "--validate", "--no_progress",
                            "nai_shuffle_work_distribution_one_to_one", lp, lp, cwd=tmp_path)
     assert rc == 0, err
     header, row = (tmp_path / "t3.csv").read_text().strip().splitlines()
     warps, chunk, dist = row.split(",")[-3:]
-    assert (warps, dist) == ("8", "rectangle") and 1 <= int(chunk) < 10, row
+    assert (warps, chunk, dist) == ("8", "40", "none"), row
+    # ... a larger one is cut into chunks of rows
+    big = write_matrices(tmp_path / "big.csv", rng.random((1, 150, 140), dtype=np.float32))
+    rc, out, err = run_cross("run", "--args_path", args, "-b", "Algorithm", "-m", "0.001", "-t", tmp_path / "t4.csv", "--validate", "--no_progress",
+                             "nai_shuffle_work_distribution_one_to_one", big, big, cwd=tmp_path)
+    assert rc == 0, err
+    assert float(out.strip().splitlines()[1].split(",")[0]) < 1e-5
+    header, row = (tmp_path / "t4.csv").read_text().strip().splitlines()
+    warps, chunk, dist = row.split(",")[-3:]
+    assert warps == "8" and dist in ("rectangle", "triangle") and 1 <= int(chunk) < 150, row
 
 
 def test_tuning_integers_select_tiles(tmp_path, oracle):

@@ -54,10 +54,12 @@ ONE_TO_ONE_CASES = [
     ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="rectangle", rows_per_thread=3)),
     ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution", distribution_type="triangle", rows_per_thread=5)),
     ("shuffle", {}),
-    ("shuffle", dict(warps_per_thread_block=4)),
+    ("shuffle", dict(whole_pair_in_lds=2)),
+    ("shuffle", dict(warps_per_thread_block=4, whole_pair_in_lds=2)),
     ("shuffle", dict(distribution_type="none")),
     ("split_row", {}),
-    ("split_row", dict(distribution_type="none")),
+    ("split_row", dict(whole_pair_in_lds=2)),
+    ("split_row", dict(distribution_type="none", whole_pair_in_lds=2)),
     ("split_row", dict(distribution_type="none", column_chunks=3)),
     ("split_row", dict(distribution_type="triangle", rows_per_thread=6, column_chunks=2)),
     ("warp_per_overlap", dict(warp_per_overlap_variant="work_distribution")),
@@ -73,10 +75,13 @@ ONE_TO_ONE_CASES = [
     ("grouped_overlap", dict(shifts_per_thread=8, rows_per_thread=16)),
     ("grouped_overlap", dict(shifts_per_thread=4, rows_per_thread=7, distribution_type="rectangle")),
     ("multimat_right", {}),
+    ("multimat_right", dict(whole_pair_in_lds=2)),
     ("multimat_right_grouped", {}),
     ("multimat_both", {}),
+    ("multimat_both", dict(whole_pair_in_lds=2)),
     ("multimat_both_grouped", {}),
     ("warp_per_overlap_lds", {}),
+    ("warp_per_overlap_lds", dict(whole_pair_in_lds=2)),
     ("warp_per_overlap_lds", dict(shifts_per_thread_block=32, shared_mem_rows=32)),
     ("warp_per_overlap_lds", dict(shifts_per_thread_block=3, shared_mem_rows=7)),
     ("warp_per_overlap_lds", dict(shifts_per_thread_block=8, column_group_per_block=1)),
@@ -150,14 +155,105 @@ def test_whole_pair_in_lds(oracle, dtype):
     assert err.value.code == 1
 
 
+def run_as_planned(xc, family, left, right, n_results, n_left, n_right, params):
+    """What a caller that asks first does: a planning call, then the launch into an output that is zeroed only when the
+    record says that the launch adds into it (filled with a NaN pattern otherwise). Returns (result, record)."""
+    rows, cols = left.shape[-2:]
+    out_shape = (n_results, 2 * rows - 1, 2 * cols - 1)
+    d_left, d_right = xc.DeviceBuffer.from_numpy(left), xc.DeviceBuffer.from_numpy(right)
+    d_out = xc.DeviceBuffer(int(np.prod(out_shape)) * left.dtype.itemsize)
+    try:
+        assert xc.lib().xcorr_plan_only(1) == 0
+        try:
+            xc.launch(family, d_left, d_right, d_out, cols, rows, n_left, n_right, left.dtype, params)
+            planned = xc.last_launch()
+        finally:
+            xc.lib().xcorr_plan_only(0)
+        if planned["uses_atomics"]:
+            d_out.zero()
+        else:
+            d_out.fill_bytes(0xFF)
+        xc.launch(family, d_left, d_right, d_out, cols, rows, n_left, n_right, left.dtype, params)
+        xc.sync()
+        rec = xc.last_launch()
+        assert rec["kernel"] == planned["kernel"] and rec["uses_atomics"] == planned["uses_atomics"] and rec["grid"] == planned["grid"]
+        return d_out.to_numpy(out_shape, left.dtype), rec
+    finally:
+        d_left.free()
+        d_right.free()
+        d_out.free()
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_few_small_pairs_whole_in_lds(oracle, dtype):
+    """The one-output-row families on few small matrices with no tile or chunk named: every pair whole in LDS, one launch,
+    plain stores into an output that nobody zeroed - one pair, one left against many, groups, all pairs; ragged shapes, more
+    pairs than the device has CUs for a block each is not possible (at most 64 pairs), a count of pairs that does not divide
+    the CUs is. A named chunk, more pairs or larger matrices keep the engine, and the planning call says which."""
+    xc = load_package()
+    rng = np.random.default_rng(777)
+    wd = dict(warp_per_overlap_variant="work_distribution")
+    one_pair = [("shuffle", {}), ("split_row", {}), ("split_row", dict(distribution_type="triangle")), ("multimat_right", {}),
+                ("multimat_right", dict(distribution_type="rectangle")), ("multimat_both", {}), ("warp_per_overlap", wd),
+                ("warp_per_overlap", dict(shifts_per_thread_block=8, distribution_type="rectangle", **wd))]
+    for family, kw in one_pair:
+        for shape in [(1, 1), (3, 5), (16, 16), (33, 17), (64, 64), (31, 97)]:
+            say("one small pair", family, kw, np.dtype(dtype).name, shape)
+            left, right = ints(rng, (1,) + shape, dtype), ints(rng, (1,) + shape, dtype)
+            got, rec = run_as_planned(xc, family, left, right, 1, 1, 1, xc.make_params(**kw))
+            assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
+            check(got, oracle.one_to_one(left[0], right[0]), True, f"{family} {kw} {shape}")
+    for shape, counts in [((16, 16), [(1, 2), (1, 32), (4, 4), (7, 9), (64, 1), (3, 1)]), ((32, 32), [(1, 8), (2, 8), (4, 4), (5, 3)]),
+                          ((13, 7), [(1, 5), (6, 6)]), ((1, 1), [(2, 2)]), ((32, 9), [(3, 7)])]:
+        for n_left, n_right in counts:
+            say("few small pairs", np.dtype(dtype).name, shape, n_left, n_right)
+            left = rng.standard_normal((n_left,) + shape).astype(dtype)
+            right_all = rng.standard_normal((n_left * n_right,) + shape).astype(dtype)
+            left_i, right_i = ints(rng, left.shape, dtype), ints(rng, right_all.shape, dtype)
+            for l, r, exact in ((left_i, right_i, True), (left, right_all, False)):
+                # groups: left l against its own n_right right matrices
+                exp = np.concatenate([oracle.one_to_many(l[i:i + 1], r[i * n_right:(i + 1) * n_right]) for i in range(n_left)])
+                family = "multimat_right_groups" if n_left > 1 else "multimat_right"
+                for kw in ({}, dict(distribution_type="triangle")):
+                    got, rec = run_as_planned(xc, family, l, r, n_left * n_right, n_left, n_right, xc.make_params(**kw))
+                    assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
+                    check(got, exp, exact, f"{family} {kw} {n_left}x{n_right} {shape}")
+                # all pairs: every left against the first n_right right matrices
+                exp = oracle.n_to_m(l, r[:n_right])
+                got, rec = run_as_planned(xc, "multimat_both", l, r[:n_right], n_left * n_right, n_left, n_right, xc.make_params())
+                assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
+                check(got, exp, exact, f"multimat_both {n_left}x{n_right} {shape}")
+    # what keeps the engine: a chunk or a tile named, whole_pair_in_lds = 2, more than 64 pairs, matrices beyond 32 x 32
+    left, right = ints(rng, (8, 16, 16), dtype), ints(rng, (72, 16, 16), dtype)
+    for family, n_left, n_right, kw in [("multimat_both", 8, 8, dict(rows_per_thread=8)), ("multimat_both", 8, 8, dict(whole_pair_in_lds=2)),
+                                        ("multimat_both", 8, 8, dict(left_matrices_per_thread=2)), ("multimat_both", 8, 9, {}),
+                                        ("multimat_right", 1, 72, {}), ("multimat_right", 1, 8, dict(right_matrices_per_thread=2))]:
+        got, rec = run_as_planned(xc, family, left[:n_left], right[:n_right], n_left * n_right, n_left, n_right, xc.make_params(**kw))
+        assert "pair_in_lds" not in rec["kernel"], (family, kw, rec)
+        exp = oracle.n_to_m(left[:n_left], right[:n_right])
+        check(got, exp, True, f"engine {family} {kw}")
+    for shape, n in [((40, 40), 2), ((32, 32), 8)]:  # (64 pairs of 32x32 are more work than the whole-pair kernel is good for)
+        left, right = ints(rng, (n,) + shape, dtype), ints(rng, (n,) + shape, dtype)
+        got, rec = run_as_planned(xc, "multimat_both", left, right, n * n, n, n, xc.make_params())
+        assert "pair_in_lds" not in rec["kernel"]
+        check(got, oracle.n_to_m(left, right), True, f"engine {shape} {n}x{n}")
+    # the LDS-staged wavefront-per-overlap family: the same route while none of its staging parameters is named
+    left, right = ints(rng, (1, 24, 24), dtype), ints(rng, (8, 24, 24), dtype)
+    for kw, routed in [({}, True), (dict(right_matrices_per_block=2), False), (dict(column_group_per_block=1), False), (dict(whole_pair_in_lds=2), False)]:
+        got, rec = run_as_planned(xc, "warp_per_overlap_lds", left, right, 8, 1, 8, xc.make_params(**kw))
+        assert ("pair_in_lds" in rec["kernel"]) == routed, (kw, rec)
+        check(got, oracle.one_to_many(left, right), True, f"warp_per_overlap_lds {kw}")
+
+
 ONE_TO_MANY_CASES = [
     ("multimat_right", {}),
+    ("multimat_right", dict(whole_pair_in_lds=2)),
     ("multimat_right", dict(right_matrices_per_thread=1)),
     ("multimat_right", dict(right_matrices_per_thread=8, warps_per_thread_block=4)),
     ("multimat_right", dict(right_matrices_per_thread=2, rows_per_thread=10, distribution_type="rectangle")),
     ("multimat_right", dict(right_matrices_per_thread=4, rows_per_thread=3, distribution_type="triangle")),
-    ("multimat_right", dict(distribution_type="none")),
-    ("multimat_right", dict(distribution_type="triangle")),
+    ("multimat_right", dict(distribution_type="none", whole_pair_in_lds=2)),
+    ("multimat_right", dict(distribution_type="triangle", whole_pair_in_lds=2)),
     ("multimat_right", dict(rows_per_thread=1, distribution_type="none")),
     ("multimat_right_grouped", {}),
     ("multimat_right_grouped", dict(shifts_per_thread_right_matrix=4, right_matrices_per_thread=4, left_rows_per_iteration=4)),
@@ -268,7 +364,8 @@ def test_many_left_matrices_with_few_right_ones_each(oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("kw", [{}, dict(distribution_type="none"), dict(right_matrices_per_thread=4, distribution_type="rectangle"),
+@pytest.mark.parametrize("kw", [{}, dict(whole_pair_in_lds=2), dict(distribution_type="none", whole_pair_in_lds=2),
+                                dict(right_matrices_per_thread=4, distribution_type="rectangle"),
                                 dict(right_matrices_per_thread=2, rows_per_thread=5, distribution_type="triangle"),
                                 dict(rows_per_thread=1, distribution_type="none")], ids=lambda v: str(v).replace(" ", ""))
 def test_multimat_right_groups(oracle, dtype, kw):
@@ -290,6 +387,7 @@ def test_multimat_right_groups(oracle, dtype, kw):
 
 N_TO_M_CASES = [
     ("multimat_both", {}),
+    ("multimat_both", dict(whole_pair_in_lds=2)),
     ("multimat_both", dict(left_matrices_per_thread=2, right_matrices_per_thread=2, rows_per_thread=10, distribution_type="triangle")),
     ("multimat_both", dict(left_matrices_per_thread=8, right_matrices_per_thread=8, rows_per_thread=3, distribution_type="rectangle")),
     ("multimat_both", dict(left_matrices_per_thread=1, right_matrices_per_thread=1, distribution_type="none")),

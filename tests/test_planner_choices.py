@@ -141,13 +141,25 @@ def test_one_row_families_on_matrix_core_tiles(plan):
     rec = plan("split_row", 256, 256, rows_per_thread=32, distribution_type="rectangle")
     assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 32 and rec["distribution_type"] == 3
     rec = plan("split_row", 256, 256, distribution_type="none")
-    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 256 and rec["uses_atomics"] == 1
+    # (one work item per result tile: plain stores, and the record says that nothing is added into the output)
+    assert rec["matrix_cores"] == 1 and rec["rows_per_worker"] == 256 and rec["uses_atomics"] == 0
     # short chunks of rows fixed by the caller, a tile request, small launches, matrix_cores = 2: the one-row tiles
     assert plan("split_row", 256, 256, rows_per_thread=7)["matrix_cores"] == 0
     assert plan("multimat_right", 128, 128, 1, 32, right_matrices_per_thread=4)["matrix_cores"] == 0
-    assert plan("shuffle", 32, 32)["matrix_cores"] == 0 and plan("shuffle", 64, 64)["matrix_cores"] == 1
-    assert plan("multimat_both", 32, 32, 2, 2)["matrix_cores"] == 0 and plan("multimat_both", 32, 32, 8, 8)["matrix_cores"] == 1
-    assert plan("multimat_right", 32, 32, 1, 2)["matrix_cores"] == 0 and plan("multimat_right", 32, 32, 1, 32)["matrix_cores"] == 1
+    # (whole_pair_in_lds = 2: not the kernel that keeps small pairs whole in LDS, which comes before the engine's tiles)
+    assert plan("shuffle", 32, 32, whole_pair_in_lds=2)["matrix_cores"] == 0 and plan("shuffle", 64, 64, whole_pair_in_lds=2)["matrix_cores"] == 1
+    assert plan("multimat_both", 32, 32, 2, 2, whole_pair_in_lds=2)["matrix_cores"] == 0
+    assert plan("multimat_both", 32, 32, 8, 8, whole_pair_in_lds=2)["matrix_cores"] == 1
+    assert plan("multimat_right", 32, 32, 1, 2, whole_pair_in_lds=2)["matrix_cores"] == 0
+    assert plan("multimat_right", 32, 32, 1, 32, whole_pair_in_lds=2)["matrix_cores"] == 1
+    # few small pairs and nothing named: every pair whole in LDS, plain stores under any of the contracts
+    for family, shape in (("shuffle", (64, 64)), ("split_row", (96, 96)), ("multimat_right", (32, 32, 1, 16)), ("multimat_right_groups", (16, 16, 4, 4)),
+                          ("multimat_both", (16, 16, 8, 8)), ("warp_per_overlap_lds", (32, 32, 1, 8))):
+        rec = plan(family, *shape)
+        assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, (family, rec)
+    assert "pair_in_lds" not in plan("multimat_both", 16, 16, 9, 8)["kernel"] and "pair_in_lds" not in plan("multimat_both", 32, 32, 8, 8)["kernel"]
+    assert "pair_in_lds" not in plan("warp_per_overlap_lds", 32, 32, 1, 8, right_matrices_per_block=2)["kernel"] and "pair_in_lds" not in plan("split_row", 128, 128)["kernel"]
+    assert "pair_in_lds" not in plan("multimat_both", 32, 32, 2, 2, rows_per_thread=8)["kernel"]
     assert plan("multimat_right", 256, 256, 1, 32, matrix_cores=2)["matrix_cores"] == 0
     # the plain launcher told to keep the rows whole keeps the summation order of one pass over the rows: a one-row tile
     rec = plan("shuffle", 256, 256, distribution_type="none")
