@@ -26,16 +26,16 @@ PEAK_TFLOPS = {"float32": 157.3, "float64": 78.6}
 # (hardware counters need the profiler around the process): the JSON says so with "traffic_measured_in_run": false.
 # Keyed by (workload, kernel of the launch record): a default launch that picks another tile reports null.
 MEASURED_TRAFFIC = {
-    ("C1", "grouped_overlap/pair_in_lds_f32_a1"): (0.32e6 + 0.18e6, "profiles/pair_in_lds_one_to_one_64.md"),
-    ("C2", "grouped_overlap/f32_m32x32"): (2.339e9 + 0.337e9, "profiles/mfma_kernel_f32_m32x32_one_to_one_1024.md"),
+    ("C1", "grouped_overlap/pair_in_lds_f32_a1"): (0.34e6 + 0.18e6, "profiles/pair_in_lds_one_to_one_64.md"),
+    ("C2", "grouped_overlap/f32_m32x32"): (2.134e9 + 0.339e9, "profiles/mfma_kernel_f32_m32x32_one_to_one_1024.md"),
     ("C2", "grouped_overlap/f32_a8b4"): (2.360e9 + 0.703e9, "profiles/engine_f32_a8b4_one_to_one_1024.md"),
-    ("C3", "multimat_right_grouped/f32_m16x16_r4"): (0.0230e9 + 0.1426e9, "profiles/engine_other_workloads.md"),
-    ("C4", "multimat_right_grouped/f32_m16x16_r4"): (0.0117e9 + 0.0673e9, "profiles/engine_other_workloads.md"),
+    ("C3", "multimat_right_grouped/f32_m16x16_r4"): (0.0191e9 + 0.1318e9, "profiles/engine_other_workloads.md"),
+    ("C4", "multimat_right_grouped/f32_m16x16_r4"): (0.0107e9 + 0.0607e9, "profiles/engine_other_workloads.md"),
     ("C3", "multimat_right_grouped/f32_m32x8_r4"): (0.0192e9 + 0.0927e9, "profiles/engine_other_workloads.md"),
     ("C4", "multimat_right_grouped/f32_m32x8_r4"): (0.0106e9 + 0.0494e9, "profiles/engine_other_workloads.md"),
     ("C3", "multimat_right_grouped/f32_a8b4_lr8"): (0.0253e9 + 0.1430e9, "profiles/engine_other_workloads.md"),
     ("C4", "multimat_right_grouped/f32_a8b4_lr8"): (0.0114e9 + 0.0619e9, "profiles/engine_other_workloads.md"),
-    ("C5", "multimat_both_grouped/f64_m8x8_l4r4"): (0.0057e9 + 0.1067e9, "profiles/engine_other_workloads.md"),
+    ("C5", "multimat_both_grouped/f64_m8x8_l4r4"): (0.0056e9 + 0.1069e9, "profiles/engine_other_workloads.md"),
     ("C5", "multimat_both_grouped/f64_a8b4_ll4lr8"): (0.0070e9 + 0.1100e9, "profiles/engine_other_workloads.md"),
 }
 
