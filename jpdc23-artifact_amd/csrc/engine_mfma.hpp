@@ -34,11 +34,12 @@
 
 namespace xcorr {
 
-// The instruction of an element type and the layout of its result tile.
-template <typename T>
+// The instruction of an element type and the layout of its result tile. FINE = 1 takes the smaller fp32 instruction (half the FMAs per
+// instruction at the same rate per cycle): tiles of 16 x 16 shifts for the sweep that trims every result tile to its own overlap.
+template <typename T, int FINE = 0>
 struct MfmaOp;
 template <>
-struct MfmaOp<float> {
+struct MfmaOp<float, 0> {
     typedef float acc_t __attribute__((ext_vector_type(16)));
     static constexpr int P = 32, ACC = 16, EV = 4;
     static constexpr int REG_BITS = 0b11011, LANE_BITS = 0b00100; // which bits of a result row come from the element index / the lane
@@ -46,13 +47,23 @@ struct MfmaOp<float> {
     static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
 };
 template <>
-struct MfmaOp<double> {
+struct MfmaOp<float, 1> { // v_mfma_f32_16x16x4_f32: 32 cycles, four k slots; element r of lanes l / 16 = kk is result row 4 kk + r
+    typedef float acc_t __attribute__((ext_vector_type(4)));
+    static constexpr int P = 16, ACC = 4, EV = 4;
+    static constexpr int REG_BITS = 0b0011, LANE_BITS = 0b1100;
+    static __device__ __forceinline__ int row(int r, int kk) { return 4 * kk + r; }
+    static __device__ __forceinline__ acc_t mma(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+};
+template <>
+struct MfmaOp<double, 0> {
     typedef double acc_t __attribute__((ext_vector_type(4)));
     static constexpr int P = 16, ACC = 4, EV = 2;
     static constexpr int REG_BITS = 0b1100, LANE_BITS = 0b0011;
     static __device__ __forceinline__ int row(int r, int kk) { return 4 * r + kk; }
     static __device__ __forceinline__ acc_t mma(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
 };
+template <>
+struct MfmaOp<double, 1> : MfmaOp<double, 0> {};
 
 constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 1); }
 
@@ -68,11 +79,16 @@ constexpr int popcount_c(int x) { return x == 0 ? 0 : (x & 1) + popcount_c(x >> 
 // P / JYO_ x shifts by IY * JYO_ y shifts of one left matrix instead of P by IY (a squarer tile sweeps fewer rows and columns that
 // only some of its shifts overlap). The copies come from the same LDS band, IY rows further down: they cost (JYO_ - 1) * IY
 // more rows per band and per chunk of left rows, no staging.
-template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int NC_ = 1, int WZ_ = 4, int JYO_ = 1>
+// FINE_: the sweep of a stage goes result tile by result tile of the wavefront, each over the rows and column steps that ITS shifts
+// overlap, instead of all tiles over the union (mfma_stage_fine): the zeros a block multiplies at the edges of the matrices are those
+// of a footprint of one result tile (P x P shifts), the work items (staging, epilogue, queue draws) those of the whole block tile.
+// For launches whose matrices are small against the block tile and share nothing between pairs.
+template <typename T, int JV_, int IU_, int MJX_, int MJV_, int NIY_, int NIU_, int RL_, int KBX_, int MINB_, int NC_ = 1, int WZ_ = 4, int JYO_ = 1,
+          int FINE_ = 0>
 struct MfmaCfg {
     using value_type = T;
-    using Op = MfmaOp<T>;
-    static constexpr int MFMA = 1, PG = 0, DB = 0;
+    using Op = MfmaOp<T, FINE_>;
+    static constexpr int MFMA = 1, PG = 0, DB = 0, FINE = FINE_;
     static constexpr int P = Op::P, ACC = Op::ACC, KS = 64 / P;
     static constexpr int VK = 16 / (int)sizeof(T);
     static constexpr int EV = Op::EV;   // consecutive elements a lane reads per operand and step = instructions per step and result tile
@@ -146,9 +162,10 @@ struct MfmaCfg {
     static constexpr int BAND_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
     static constexpr int LDS_BYTES = BAND_BYTES + 16; // + two slots through which thread 0 hands the block its next work item
     static_assert(P % (JV * JYO) == 0 && P % IU == 0, "whole matrices per result tile");
+    static_assert(FINE == 0 || (JV == 1 && IU == 1 && JYO == 1 && MJV == 1 && NIU == 1), "tile-by-tile sweep: the result tiles of a block are shifts of one pair");
     static_assert(JYO == 1 || (JV == 1 && NIY == 1), "copies of the x shifts: one left matrix per result tile, one tile along y");
     static_assert(EV % NC == 0, "the instructions of a step are dealt evenly to the accumulator sets");
-    static_assert(WZ > 1 && (KBX / K) % WZ == 0, "every wavefront gets the same number of column chunks per stage");
+    static_assert(WZ > 1 && (FINE != 0 ? KBX % K == 0 : (KBX / K) % WZ == 0), "every wavefront gets the same number of column chunks per stage");
     static_assert((PV % VK == 0 || JYO > 1) && VBAND % VK == 0 && UBAND % VK == 0, "128-bit LDS pieces");
     static_assert(LX * LY * LV * LU * WY == 64, "lane bookkeeping");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
@@ -428,6 +445,104 @@ __device__ __forceinline__ void mfma_stage(const typename C::value_type *Vs_lane
     }
 }
 
+// The same for a FINE tile: the wavefront's result tiles (s along x, t along y) are swept one after the other, tile (s, t) over the
+// column steps [ka_s, kb_s) and rows [ja_t, ja_t + nt_t) of the stage that its own P x P shifts overlap. The (step, tile, row) triples of
+// the stage are numbered row-fastest and cut into WZ equal runs, one per wavefront.
+// Stage geometry: its first right column is x0, its first base row yl0; the block tile's first shifts are (sxb, syb); the work item
+// holds the right columns below w_hi and the left rows below chi.
+template <class C>
+__device__ __forceinline__ void mfma_stage_fine(const typename C::value_type *Vs_lane, const typename C::value_type *Us_lane,
+                                                typename C::Op::acc_t (&acc)[C::TJ][C::TI][C::NC], int wave, int x0, int sxb, int W, int w_hi,
+                                                int yl0, int syb, int H, int chi) {
+    using T = typename C::value_type;
+    typedef T evec __attribute__((ext_vector_type(C::EV)));
+    constexpr int EV = C::EV, K = C::K, NKC = C::KBX / C::K;
+    // rows of tile t: base rows yb = yl0 + j whose window meets the right matrix, yb in [syb + t IY, syb + t IY + IY - 1 + H - 1], yb < chi
+    int ja[C::TI], nt[C::TI], rows_all = 0;
+#pragma unroll
+    for (int t = 0; t < C::TI; ++t) {
+        const int first = syb + t * C::IY - yl0;
+        int last = first + C::IY + H - 2;
+        if (chi - 1 - yl0 < last) last = chi - 1 - yl0;
+        if (last > C::RL - 1) last = C::RL - 1;
+        ja[t] = first > 0 ? first : 0;
+        nt[t] = last + 1 - ja[t] > 0 ? last + 1 - ja[t] : 0;
+        rows_all += nt[t];
+    }
+    // column steps of tile s (x shifts sxb + s JX ...): (x0 + kc K + K - 1) + (sx + JX - 1) >= 0, (x0 + kc K) + sx <= W - 1, x0 + kc K < w_hi
+    int ka[C::TJ], kb[C::TJ], steps_all = 0;
+#pragma unroll
+    for (int s = 0; s < C::TJ; ++s) {
+        const int sx = sxb + s * C::JX;
+        const int need = -(sx + C::JX - 1) - (K - 1) - x0;
+        ka[s] = need > 0 ? (need + K - 1) / K : 0;
+        int lim = W - 1 - sx - x0;
+        if (w_hi - 1 - x0 < lim) lim = w_hi - 1 - x0;
+        kb[s] = lim < 0 ? 0 : lim / K + 1;
+        if (kb[s] > NKC) kb[s] = NKC;
+        if (kb[s] < ka[s]) kb[s] = ka[s];
+        steps_all += kb[s] - ka[s];
+    }
+    const int total = steps_all * rows_all;
+    const int lo = total * wave / C::WZ, hi = total * (wave + 1) / C::WZ; // this wavefront's run [lo, hi)
+    if (lo >= hi) return;
+    int pos = 0;
+#pragma unroll 1
+    for (int kc = 0; kc < NKC; ++kc) {
+#pragma unroll
+        for (int s = 0; s < C::TJ; ++s) {
+            if (kc < ka[s] || kc >= kb[s]) continue;
+#pragma unroll
+            for (int t = 0; t < C::TI; ++t) {
+                const int begin = (lo > pos ? lo : pos) - pos, end = (hi < pos + nt[t] ? hi : pos + nt[t]) - pos;
+                pos += nt[t];
+                if (begin >= end) continue;
+                const int j0 = __builtin_amdgcn_readfirstlane(ja[t] + begin), n = __builtin_amdgcn_readfirstlane(end - begin);
+                const T *vp = Vs_lane + kc * K + j0 * C::PV + s * C::JX;
+                const T *up = Us_lane + kc * K + j0 * C::PU - t * C::IY * C::PU;
+                auto load = [](const T *v, const T *u, evec &a, T (&b)[EV]) __attribute__((always_inline)) {
+                    a = *reinterpret_cast<const evec *>(u);
+#pragma unroll
+                    for (int e = 0; e < EV; ++e) b[e] = v[e];
+                };
+                auto multiply = [&](const evec &a, const T (&b)[EV]) __attribute__((always_inline)) {
+#pragma unroll
+                    for (int e = 0; e < EV; ++e) acc[s][t][e % C::NC] = C::Op::mma(a[e], b[e], acc[s][t][e % C::NC]);
+                };
+                // (as in mfma_stage: the reads of the next row before the instructions of the current one, four rows per trip; the read
+                // past the last row lands in the spare row of the bands)
+                evec a0, a1;
+                T b0[EV], b1[EV];
+                load(vp, up, a0, b0);
+                int j = 0;
+#pragma unroll 1
+                for (; j + 4 <= n; j += 4) {
+                    load(vp + C::PV, up + C::PU, a1, b1);
+                    multiply(a0, b0);
+                    load(vp + 2 * C::PV, up + 2 * C::PU, a0, b0);
+                    multiply(a1, b1);
+                    load(vp + 3 * C::PV, up + 3 * C::PU, a1, b1);
+                    multiply(a0, b0);
+                    vp += 4 * C::PV;
+                    up += 4 * C::PU;
+                    load(vp, up, a0, b0);
+                    multiply(a1, b1);
+                }
+#pragma unroll 1
+                for (; j + 2 <= n; j += 2) {
+                    load(vp + C::PV, up + C::PU, a1, b1);
+                    multiply(a0, b0);
+                    vp += 2 * C::PV;
+                    up += 2 * C::PU;
+                    load(vp, up, a0, b0);
+                    multiply(a1, b1);
+                }
+                if (j < n) multiply(a0, b0);
+            }
+        }
+    }
+}
+
 // One block = four wavefronts that take work items one after the other. A launch is either one block per work item
 // (gridDim.x = total_items, g.queue == nullptr) or PERSISTENT: as many blocks as the device holds at a time, each taking its own
 // index as first item and every further one from the launch's queue counter (g.queue), i.e. in launch order - heaviest first -
@@ -474,12 +589,6 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
         left_band.init(tid, W);
     right_dma.init(lane, group, W);
 
-#ifdef XCORR_EXP_STAGGER
-    if (g.queue != nullptr) {
-        const int phase = (int)(blockIdx.x * 4 / gridDim.x);
-        for (int i = 0; i < phase * XCORR_EXP_STAGGER; ++i) __builtin_amdgcn_s_sleep(32); // 32 x 64 cycles
-    }
-#endif
     // The queue this block draws from; the k-th draw stands for item my_queue + gridDim.x + queues * k. (Letting a block whose
     // queue is empty draw from the others was measured: every block then ends with up to eight draws nothing hides, and all
     // five benchmark workloads ran 1-2 % slower.)
@@ -593,7 +702,10 @@ __global__ __launch_bounds__(C::NT, C::MINB) void mfma_kernel(EngineArgs<typenam
                     }
                     if (nrows > 0 && kc_hi > kc_lo) {
                         __builtin_amdgcn_s_setprio(0);
-                        mfma_stage<C>(Vs_lane, Us_lane, acc, group, kc_lo, kc_hi, row0, nrows);
+                        if constexpr (C::FINE != 0)
+                            mfma_stage_fine<C>(Vs_lane, Us_lane, acc, group, x0, sxb, W, w_hi, yl0, syb, H, chi);
+                        else
+                            mfma_stage<C>(Vs_lane, Us_lane, acc, group, kc_lo, kc_hi, row0, nrows);
                         __builtin_amdgcn_s_setprio(2);
                     }
                 }

@@ -6,13 +6,13 @@
 
 namespace xcorr {
 
-//                               T    JV IU MJX MJV NIY NIU  RL KBX MINB AL
+//                               T    JV IU MJX MJV NIY NIU  RL KBX MINB
 using D_32x32 = MfmaCfg<double, 1, 1, 2, 1, 2, 1, 32, 32, 4>;
 using D_32x16 = MfmaCfg<double, 1, 1, 2, 1, 1, 1, 32, 32, 4>;
 using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
 // (the same right matrices with 16 x 16 shifts - the columns of a result tile 8 x shifts twice, 8 left rows apart, as the fp32 file
 // has them - measured level with D_32x8_r4 from 64x64 matrices on and 6 % faster on 32x32 only: not compiled)
-// (stages of 12 rows and four pieces per staging batch: 128 registers and 40 KB of LDS, four blocks per CU; 16 rows at three blocks 2 % slower,
+// (stages of 12 rows: 128 registers and 40 KB of LDS, four blocks per CU; 16 rows at three blocks 2 % slower,
 // 8 rows at four blocks level with that)
 using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4>;
 

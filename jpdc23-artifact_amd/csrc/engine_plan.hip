@@ -50,6 +50,8 @@ static const struct {
     {"f32_m16x16_r4", 4},
     {"f32_m16x16_r8", 4},
     {"f32_m8x8_l4r8", 4},
+    {"f32_m32x32_s16", 7},
+    {"f32_m64x64_s16", 5},
     {"f64_a1b8", 5},
     {"f64_a1b4_l2r2", 4},
     {"f64_a8b8", 2},
@@ -251,15 +253,17 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     const double us_per_atomic = mm ? (lanes_over_matrices ? (f32 ? 1.98e-6 : 3.06e-6) : (f32 ? 2.37e-6 : 1.51e-6))
                                     : lanes_over_matrices ? (f32 ? 4.5e-6 : 3.0e-6) : (f32 ? 1.6e-6 : 4.4e-6);
     const double cyc = (f32 ? 2.0 : 4.0) / 2100.0; // microseconds per FMA instruction of a wavefront
-    const double W = rq.W, H = rq.H, TXW = s.TXB(), TYW = s.TYB();
+    // (a tile-by-tile sweep pays the edge zeros of one result tile, not of the block tile)
+    const double W = rq.W, H = rq.H, TXW = s.fine_x ? s.fine_x : s.TXB(), TYW = s.fine_y ? s.fine_y : s.TYB();
+    const double ntx = (double)plan.ntx * s.TXB() / TXW, nty = (double)plan.nty * s.TYB() / TYW;
     const bool split = plan.atomic != 0 || plan.ordered;
     const double rc = plan.rows_per_chunk;
     // a tile overlaps cols_tile right columns on average; cut into chunks, ceil(cols_tile / chunk) of its
     // x_chunks work items find columns, the others return at once
-    const double cols_tile = std::fmin(W, W * (W + TXW) / (plan.ntx * TXW));
+    const double cols_tile = std::fmin(W, W * (W + TXW) / (ntx * TXW));
     const double live = plan.x_chunks > 1 ? std::fmin(plan.x_chunks, std::ceil(cols_tile / plan.x_chunk_cols)) : 1.0;
     const double cols_avg = cols_tile / live, cols_max = plan.x_chunks > 1 ? std::fmin(W, plan.x_chunk_cols) : W;
-    const double rows_tile = std::fmin(H, H * (H + TYW) / (plan.nty * TYW));
+    const double rows_tile = std::fmin(H, H * (H + TYW) / (nty * TYW));
     const double rows_avg = (split && rc < rows_tile ? rc + copies : rows_tile) + window;
     const double rows_max = (split && rc < H ? rc + copies : H + 0.5 * copies) + window;
     const double per_element = (double)s.NV * s.NU * s.A * s.B / s.WZ * s.issue_factor;
@@ -323,6 +327,11 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
             // The tiles whose columns hold copies of the x shifts win up to about 256x256 matrices (2-7 % over their 32 x 8
             // counterparts) and measured level at 300x300, 3-14 % behind at 384x384 ... 1024x1024, which the model does not show.
             if (s.MFMA && s.TYB() != s.TYW() && (double)rq.W * rq.H > 300.0 * 300.0) continue;
+            // The tile-by-tile sweep is the launcher's own choice (a request for y shifts per thread means the tiles that had them
+            // before), for matrices of 17 ... 300 rows and columns: on 16x16 the four-shift register tile is ahead (30 against 36 us
+            // for 4000 pairs), one pair of 512x512 runs 8 % slower than on the 32 x 32 tile (its edge is a small share there, and
+            // the smaller instruction issues twice as often), 1024x1024 level.
+            if (s.fine_y && (rq.y_shifts > 1 || (rq.W <= 16 && rq.H <= 16) || (double)rq.W * rq.H > 300.0 * 300.0)) continue;
             if (rq.x_shifts && (unsigned)s.B != rq.x_shifts) continue;
             if (rq.lanes_x && (unsigned)s.LX != rq.lanes_x) continue;
             if (rq.lanes_y && (unsigned)s.LY != rq.lanes_y) continue;
@@ -333,12 +342,15 @@ static int plan_grouped(const EngineRequest &rq, const EngineSpec *specs, int co
         const int longest = rq.W > rq.H ? rq.W : rq.H;
         const bool no_request = rq.spec_index == 0 && rq.y_shifts == 0 && rq.left_mats <= 1 && rq.right_mats == 0 && rq.x_shifts == 0 &&
                                 rq.lanes_x == 0 && rq.lanes_y == 0;
-        if (no_request && s.A > 4 && (longest <= (s.PG ? 16 : 24) || (longest <= 32 && !s.PG && (rq.group_m > 0 || rq.nV == 1)))) continue;
+        if (no_request && s.A > 4 && !s.fine_x && (longest <= (s.PG ? 16 : 24) || (longest <= 32 && !s.PG && (rq.group_m > 0 || rq.nV == 1)))) continue;
         const RequestMatch match = match_request(s, rq);
         if (found && best_match.better_than(match)) continue;
         const int G = s.MFMA ? 8 : s.A + 1; // granule of the chunk sizes tried
         const bool matrices_in_tile = s.MFMA ? s.NVB() * s.NUB() > 1 : s.LV * s.LU > 1;
         for (int k : ladder) {
+            // (chunks of rows leave the trimming of a tile's rows nothing to save: one pair of 256x256 in chunks of 32 rows measured 8 %
+            // slower than on the 32 x 32 tile)
+            if (k != 0 && s.fine_y && rq.rows_per_worker == 0) break;
             int rc = k * G;
             if (rq.rows_per_worker > 0) {
                 if (k != 0) break;

@@ -34,6 +34,8 @@ struct EngineSpec {
     // useful FMA instruction (LDS reads, waits and address arithmetic included), and the relative cost
     // of staging one band
     double issue_factor, stage_factor;
+    // matrix-core tiles whose sweep trims every result tile of a block to its own overlap: the shifts of one result tile (else 0)
+    int fine_x, fine_y;
     // the same, with the figure of an MI355X where no device can be asked (planning without a GPU)
     int resident_blocks() const;
     int TXW() const { return LX * B; }
@@ -54,16 +56,9 @@ constexpr auto kernel_of() {
         return &engine_kernel<C>;
 }
 
-// EXPERIMENT: dynamic LDS size override
-template <class C>
-int exp_lds() {
-    static int v = -1;
-    if (v < 0) { const char *e = getenv("XCORR_EXP_LDS"); v = e ? atoi(e) : 0; }
-    return C::MFMA && v > C::LDS_BYTES ? v : C::LDS_BYTES;
-}
 template <class C>
 hipError_t allow_large_lds() {
-    if (exp_lds<C>() <= 64 * 1024) return hipSuccess;
+    if (C::LDS_BYTES <= 64 * 1024) return hipSuccess;
     // the attribute belongs to the kernel's copy on one device: kept per device of the process
     static bool attr_set[64] = {};
     int dev = 0;
@@ -71,7 +66,7 @@ hipError_t allow_large_lds() {
     const bool tracked = dev >= 0 && dev < 64;
     if (!tracked || !attr_set[dev]) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel_of<C>()),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, exp_lds<C>());
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, C::LDS_BYTES);
         if (e != hipSuccess) return e;
         if (tracked) attr_set[dev] = true;
     }
@@ -82,7 +77,7 @@ template <class C>
 hipError_t launch_engine(const void *args, unsigned grid, hipStream_t stream) {
     using T = typename C::value_type;
     if (hipError_t e = allow_large_lds<C>(); e != hipSuccess) return e;
-    kernel_of<C>()<<<dim3(grid), dim3(C::NT), exp_lds<C>(), stream>>>(*static_cast<const EngineArgs<T> *>(args));
+    kernel_of<C>()<<<dim3(grid), dim3(C::NT), C::LDS_BYTES, stream>>>(*static_cast<const EngineArgs<T> *>(args));
     return hipGetLastError();
 }
 
@@ -93,13 +88,21 @@ int resident_blocks_engine() {
     if (blocks[dev] == 0) {
         int n = 0;
         if (allow_large_lds<C>() != hipSuccess ||
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, exp_lds<C>()) != hipSuccess || n < 1) {
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, reinterpret_cast<const void *>(kernel_of<C>()), C::NT, C::LDS_BYTES) != hipSuccess || n < 1) {
             (void)hipGetLastError();
             return 0; // (not kept: a device may appear later)
         }
         blocks[dev] = n;
     }
     return blocks[dev];
+}
+
+template <class C>
+constexpr int fine_extent(bool along_x) {
+    if constexpr (C::MFMA != 0) {
+        if constexpr (C::FINE != 0) return along_x ? C::JX : C::IY;
+    }
+    return 0;
 }
 
 template <class C>
@@ -113,7 +116,8 @@ constexpr EngineSpec make_spec(const char *name, double issue_factor = 1.0, doub
                       C::WY,  C::RL,
                       C::KBX, C::WZ,
                       C::PG,  C::MFMA, C::LDS_BYTES,
-                      C::NT,  &launch_engine<C>, &resident_blocks_engine<C>, issue_factor, stage_factor};
+                      C::NT,  &launch_engine<C>, &resident_blocks_engine<C>, issue_factor, stage_factor,
+                      fine_extent<C>(true), fine_extent<C>(false)};
 }
 
 // defined in engine_f32.hip / engine_f64.hip

@@ -342,12 +342,14 @@ def test_n_to_mn_one_launch(oracle, dtype, kw):
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_many_left_matrices_with_few_right_ones_each(oracle, dtype):
     """n_to_mn with one or two right matrices per left matrix (independent pairs): no tile that lays lanes over the right
-    matrices of ONE left matrix has anything to share, the launcher's pick for thousands of 32x32 fp32 pairs is the tile
-    that lays its lanes over left matrices with their own groups; bit-exact whatever it picks."""
+    matrices of ONE left matrix has anything to share. The launcher's pick for thousands of small fp32 pairs is a matrix-core
+    tile whose sweep trims each 16 x 16 result tile to its own overlap (the register tile that lays eight lanes over left
+    matrices with their own groups is what `matrix_cores` = 2 runs); bit-exact whatever it picks."""
     xc = load_package()
     rng = np.random.default_rng(420)
     picked = set()
-    for n, m, shape in [(2000, 1, (32, 32)), (1000, 2, (32, 32)), (301, 1, (40, 36)), (77, 3, (33, 31)), (1500, 1, (20, 24))]:
+    for n, m, shape in [(2000, 1, (32, 32)), (1000, 2, (32, 32)), (301, 1, (40, 36)), (77, 3, (33, 31)), (1500, 1, (20, 24)), (500, 1, (64, 64)),
+                        (40, 1, (100, 90)), (1200, 1, (16, 16)), (900, 1, (17, 18))]:
         say("n_to_mn, few right matrices per left", np.dtype(dtype).name, n, m, shape)
         left = ints(rng, (n,) + shape, dtype)
         right = ints(rng, (n * m,) + shape, dtype)
@@ -358,9 +360,13 @@ def test_many_left_matrices_with_few_right_ones_each(oracle, dtype):
         got_dev = xc.run("multimat_right_grouped", left, right_dev, n * m, n_left=n, n_right=m)
         picked.add(xc.last_launch()["kernel"])
         check(got_dev[slot], exp, True, f"n_to_mn {n}x{m} {shape}")
+        if dtype == np.float32 and shape[0] <= 40:
+            got_dev = xc.run("multimat_right_grouped", left, right_dev, n * m, n_left=n, n_right=m, params=xc.make_params(matrix_cores=2))
+            picked.add(xc.last_launch()["kernel"])
+            check(got_dev[slot], exp, True, f"n_to_mn {n}x{m} {shape}, vector FMAs")
     say("kernels:", sorted(picked))
-    if dtype == np.float32:  # (in fp64 that tile measured slower than the single-matrix tiles and is not compiled)
-        assert any("pairs8" in k for k in picked), picked
+    if dtype == np.float32:  # (fp64 has neither: the paired tile measured slower than the single-matrix tiles there)
+        assert any("pairs8" in k for k in picked) and any("m64x64_s16" in k for k in picked) and any("m32x32_s16" in k for k in picked), picked
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
