@@ -57,3 +57,50 @@ def test_default_launches_agree_with_themselves_to_the_last_bits():
     assert d <= 1e-12
     a, b, rec = run_twice(xc, "split_row", left[:256, :256], right[:256, :256], 1, 1, 1)
     assert rec["uses_atomics"] == 1 and distance(a, b) <= 1e-6
+
+
+def test_output_in_pinned_host_memory(oracle):
+    """The float atomic add is not defined on host-mapped memory (it is dropped without an error): a launch into such an
+    output that names no chunk is replanned with whole reductions and plain stores and gives the right result; one whose
+    chunk the caller fixed is refused (XCORR_ERR_UNSUPPORTED) before anything is launched."""
+    import ctypes
+
+    xc = load_package()
+    lib = xc.lib()
+    rng = np.random.default_rng(79)
+    rows = cols = 200
+    left = rng.integers(-3, 4, (rows, cols)).astype(np.float32)
+    right = rng.integers(-3, 4, (rows, cols)).astype(np.float32)
+    out_shape = (2 * rows - 1, 2 * cols - 1)
+    exp = oracle.one_to_one(left, right).reshape(out_shape)
+    nbytes = int(np.prod(out_shape)) * 4
+    d_left, d_right = xc.DeviceBuffer.from_numpy(left), xc.DeviceBuffer.from_numpy(right)
+    host = ctypes.c_void_p()
+    assert lib.xcorr_host_alloc_pinned(ctypes.byref(host), ctypes.c_size_t(nbytes)) == 0
+    try:
+        view = np.ctypeslib.as_array(ctypes.cast(host, ctypes.POINTER(ctypes.c_float)), shape=out_shape)
+        for family, fn in (("grouped_overlap", lib.xcorr_grouped_overlap_f32), ("split_row", lib.xcorr_split_row_f32)):
+            # on device memory this launch splits and adds atomically ...
+            lib.xcorr_plan_only(1)
+            p = xc.make_params()
+            assert fn(d_left.ptr, d_right.ptr, d_left.ptr, cols, rows, ctypes.byref(p), None) == 0
+            planned = xc.last_launch()
+            lib.xcorr_plan_only(0)
+            assert planned["uses_atomics"] == 1, planned
+            # ... into pinned host memory it does not
+            view[:] = np.nan
+            code = fn(d_left.ptr, d_right.ptr, host, cols, rows, ctypes.byref(p), None)
+            assert code == 0, lib.xcorr_last_error()
+            xc.sync()
+            rec = xc.last_launch()
+            print(family, "into pinned host memory:", rec["kernel"], "atomics", rec["uses_atomics"], flush=True)
+            assert rec["uses_atomics"] == 0 and rec["rows_per_worker"] == rows
+            assert np.array_equal(view, exp), family
+            p = xc.make_params(rows_per_thread=32)
+            assert fn(d_left.ptr, d_right.ptr, host, cols, rows, ctypes.byref(p), None) == 3
+            assert b"atomics" in lib.xcorr_last_error()
+    finally:
+        xc.sync()
+        lib.xcorr_host_free(host)
+        d_left.free()
+        d_right.free()
