@@ -453,6 +453,25 @@ def main():
                 entry["parity"] = parity_against_host_loops(oracle, v.d_out.to_numpy(v.out_shape, dtype)[0], band, lo, hi, exact, lo64, hi64, dtype)
             v.free()
             per[key] = entry
+        # Thousands of independent small pairs (n-to-mn with one right matrix per left matrix: the regime of the reference's
+        # one_to_one_saturated files), where no tile can share a matrix between pairs.
+        for size in (64, 32):
+            shape = dict(mode="n_to_mn", dtype="float32", rows=size, cols=size, n_left=4000, n_right=4000, dist="uniform", seed=2023,
+                         family="multimat_right_grouped")
+            v = Workload(xc, workloads, f"n_to_mn:4000:4000:{size}", None, "{}", cfg=shape)
+            v_wall, v_ev = v.timed(20, args.warmup)
+            v_rec = xc.last_launch()
+            entry = roofline_of(v, v_rec, v_ev / 20, False)
+            entry.update({"workload": f"n_to_mn 4000x4000 of {size}x{size} float32 (one right matrix per left matrix), family {v.family}",
+                          "kernel": v_rec["kernel"], "steps": 20, "ms_per_step": round(v_wall * 1e3 / 20, 5)})
+            if oracle is not None:  # the first sixteen pairs against the oracle
+                got = v.result_in_file_order()[:16]
+                exp = np.stack([oracle.one_to_one(v.left[i], v.right[i]).reshape(got.shape[1:]) for i in range(16)])
+                e = oracle.errors(got, exp)
+                entry["parity"] = {"against": "oracle, 16 whole results", "bar": 1e-5, "rel_frobenius": float(f"{e.rel_frobenius:.3e}"),
+                                   "within_bar": bool(e.rel_frobenius <= 1e-5)}
+            v.free()
+            per[f"independent_pairs_{size}"] = entry
         result["per_config"] = per
     print(json.dumps(result))
 
