@@ -162,7 +162,7 @@ struct MfmaCfg {
     static constexpr int BAND_BYTES = (LDS_ELEMS > RED_ELEMS ? LDS_ELEMS : RED_ELEMS) * (int)sizeof(T);
     static constexpr int LDS_BYTES = BAND_BYTES + 16; // + two slots through which thread 0 hands the block its next work item
     static_assert(P % (JV * JYO) == 0 && P % IU == 0, "whole matrices per result tile");
-    static_assert(FINE == 0 || (JV == 1 && IU == 1 && JYO == 1 && MJV == 1 && NIU == 1), "tile-by-tile sweep: the result tiles of a block are shifts of one pair");
+    static_assert(FINE == 0 || (JYO == 1 && MJV == 1 && NIU == 1), "tile-by-tile sweep: the result tiles of a block differ in their shifts only");
     static_assert(JYO == 1 || (JV == 1 && NIY == 1), "copies of the x shifts: one left matrix per result tile, one tile along y");
     static_assert(EV % NC == 0, "the instructions of a step are dealt evenly to the accumulator sets");
     static_assert(WZ > 1 && (FINE != 0 ? KBX % K == 0 : (KBX / K) % WZ == 0), "every wavefront gets the same number of column chunks per stage");

@@ -34,6 +34,11 @@ using M_32x32_s16 = MfmaCfg<float, 1, 1, 2, 1, 2, 1, 32, 32, 6, 1, 4, 1, 1>;
 // four by four result tiles: a pair of up to 32x32 is one work item
 using M_64x64_s16 = MfmaCfg<float, 1, 1, 4, 1, 4, 1, 32, 32, 5, 1, 4, 1, 1>;
 // (stages of 64 columns instead of 32: 1-2 % slower on 32x32 ... 96x96 pairs with either tile; stages of 16 rows: 5 % slower on 32x32)
+// The same sweep with four right matrices in the rows of a result tile (4 y shifts each) and four result tiles down a wavefront: the 16 x 16
+// shifts of the m16x16_r4 tile above, trimmed along y to 4 shifts at a time. C4 0.641 -> 0.598 ms, C3 4.30 -> 4.19 ms, 1 x 256 of 64x64 119 -> 106 us.
+// (Stages of 32 rows at four or five blocks per CU: +0.7 %; stages of 64 columns: +17 %; two accumulator sets: level; 32 x 16 shifts per block: +5 %;
+// eight right matrices with 2 y shifts each: +13 %.)
+using M_16x16_r4_s4 = MfmaCfg<float, 1, 4, 1, 1, 4, 1, 16, 32, 5, 1, 4, 1, 1>;
 
 static const EngineSpec specs[] = {
     // (issue and staging factors of the run-time model: fitted to launches of 16x16 ... 1024x1024 matrices, 1 ... 1024 pairs)
@@ -47,6 +52,7 @@ static const EngineSpec specs[] = {
     make_spec<M_8x8_l4r8>("f32_m8x8_l4r8", 0.745, 1.0),
     make_spec<M_32x32_s16>("f32_m32x32_s16", 0.83, 1.0),
     make_spec<M_64x64_s16>("f32_m64x64_s16", 0.84, 1.0),
+    make_spec<M_16x16_r4_s4>("f32_m16x16_r4_s4", 0.68, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f32(int *count) {

@@ -16,11 +16,18 @@ using D_32x8_r4 = MfmaCfg<double, 1, 2, 2, 1, 1, 2, 16, 32, 4>;
 // 8 rows at four blocks level with that)
 using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4>;
 
+// D_32x32 with the sweep that goes result tile by result tile, each over the rows and column steps its own 16 x 16 shifts overlap
+// (engine_mfma.hpp, FINE_): for many small pairs that share nothing - 2000 independent pairs of 32x32 / 64x64 / 128x128: 0.24 / 0.45 / 0.64 ->
+// 0.32 / 0.55 / 0.71 of the fp64 peak. (The pair tile trimmed the same way, 4 x 4 shifts at a time, is 8 % SLOWER on C5: its one-tile runs are
+// bound by their LDS reads.)
+using D_32x32_s16 = MfmaCfg<double, 1, 1, 2, 1, 2, 1, 32, 32, 4, 1, 4, 1, 1>;
+
 static const EngineSpec specs[] = {
     make_spec<D_32x32>("f64_m32x32", 0.696, 1.0),
     make_spec<D_32x16>("f64_m32x16", 0.697, 1.0),
     make_spec<D_32x8_r4>("f64_m32x8_r4", 0.705, 1.0),
     make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.730, 1.0),
+    make_spec<D_32x32_s16>("f64_m32x32_s16", 0.80, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f64(int *count) {

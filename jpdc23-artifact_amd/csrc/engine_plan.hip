@@ -52,6 +52,7 @@ static const struct {
     {"f32_m8x8_l4r8", 4},
     {"f32_m32x32_s16", 7},
     {"f32_m64x64_s16", 5},
+    {"f32_m16x16_r4_s4", 6},
     {"f64_a1b8", 5},
     {"f64_a1b4_l2r2", 4},
     {"f64_a8b8", 2},
@@ -72,6 +73,7 @@ static const struct {
     {"f64_m32x16", 4},
     {"f64_m32x8_r4", 4},
     {"f64_m8x8_l4r4", 4},
+    {"f64_m32x32_s16", 4},
 };
 
 int EngineSpec::resident_blocks() const {

@@ -118,7 +118,7 @@ def test_tiles_with_copies_of_the_x_shifts(oracle):
             if "does not exist" in e.message:
                 break
             continue
-        if "_m16x16_" in xc.last_launch()["kernel"]:
+        if "_m16x16_" in xc.last_launch()["kernel"] and not xc.last_launch()["kernel"].endswith("_s4"):
             indices.append(index)
     assert len(indices) == 2, indices
     for index in indices:
@@ -200,3 +200,57 @@ def test_one_output_row_families_on_matrix_core_tiles(oracle, dtype):
         assert rec["matrix_cores"] == routed, (family, kw, rec["kernel"])
         assert np.array_equal(got, exp), (family, kw, rec["kernel"])
     say(sorted(seen))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_tiles_swept_result_tile_by_result_tile(oracle, dtype):
+    """The tiles whose sweep trims every result tile of a block to its own overlap (`_s16`: one pair, 16 x 16 shifts at a time;
+    `_r4_s4`: four right matrices, 16 x 4 shifts at a time), forced by index: shapes below, at and above the extents of a result tile
+    and of a block tile, one-row and one-column matrices, whole reductions and chunks of left rows and right columns that start
+    and end anywhere (atomic adds), one left matrix against several right ones, groups, all pairs; the launcher's own choice on
+    launches they are best for. Bit-exact on integers."""
+    xc = load_package()
+    rng = np.random.default_rng(906)
+    indices = {}
+    probe = ints(rng, (1, 4, 4), dtype)
+    for index in range(1, 80):
+        try:
+            xc.run("multimat_right_grouped", probe, probe, 1, n_left=1, n_right=1, params=xc.make_params(specialisation=index))
+        except xc.XcorrError as e:
+            if "does not exist" in e.message:
+                break
+            continue
+        kernel = xc.last_launch()["kernel"].split("/")[1]
+        if kernel.endswith("_s16") or kernel.endswith("_s4"):
+            indices[kernel] = index
+    say("tiles:", indices)
+    assert len(indices) == (3 if dtype == np.float32 else 1), indices
+    for kernel, index in indices.items():
+        for shape in [(1, 1), (1, 40), (37, 1), (5, 3), (15, 17), (16, 16), (17, 31), (32, 32), (33, 47), (64, 64), (65, 63), (70, 130), (150, 41)]:
+            for n_right in (1, 3, 4, 9) if "_r4" in kernel else (1, 2):
+                left, right = ints(rng, (1,) + shape, dtype), ints(rng, (n_right,) + shape, dtype)
+                exp = oracle.one_to_many(left, right)
+                for kw in [{}, dict(rows_per_thread=3), dict(rows_per_thread=8), dict(rows_per_thread=24), dict(rows_per_thread=40, column_chunks=2)]:
+                    got = xc.run("multimat_right_grouped", left, right, n_right, n_left=1, n_right=n_right, params=xc.make_params(specialisation=index, **kw))
+                    rec = xc.last_launch()
+                    assert rec["kernel"].endswith(kernel)
+                    bad = np.argwhere(got != exp)
+                    assert bad.size == 0, (kernel, shape, n_right, kw, bad[:3].tolist())
+        left, right = ints(rng, (3, 21, 45), dtype), ints(rng, (15, 21, 45), dtype)
+        exp = np.concatenate([oracle.one_to_many(left[l:l + 1], right[l * 5:(l + 1) * 5]) for l in range(3)])
+        assert np.array_equal(xc.run("multimat_right_grouped", left, right, 15, n_left=3, n_right=5, params=xc.make_params(specialisation=index)), exp)
+        exp = oracle.n_to_m(left, right)
+        assert np.array_equal(xc.run("multimat_both_grouped", left, right, 45, n_left=3, n_right=15, params=xc.make_params(specialisation=index, rows_per_thread=16)), exp)
+        left, right = ints(rng, (1, 100, 90), dtype), ints(rng, (1, 100, 90), dtype)
+        assert np.array_equal(xc.run("grouped_overlap", left, right, 1, params=xc.make_params(specialisation=index)), oracle.one_to_one(left[0], right[0]))
+    # the launcher's own choice: many independent pairs; one left matrix against many right ones (fp32)
+    left, right = ints(rng, (600, 48, 48), dtype), ints(rng, (600, 48, 48), dtype)
+    got = xc.run("multimat_right_grouped", left, right, 600, n_left=600, n_right=1)
+    assert xc.last_launch()["kernel"].endswith("_s16"), xc.last_launch()["kernel"]
+    assert np.array_equal(got, oracle.n_to_mn(left, right, threads=8))
+    if dtype == np.float32:
+        left, right = ints(rng, (1, 128, 128), dtype), ints(rng, (64, 128, 128), dtype)
+        got = xc.run("multimat_right_grouped", left, right, 64, n_left=1, n_right=64)
+        assert xc.last_launch()["kernel"].endswith("_r4_s4"), xc.last_launch()["kernel"]
+        sample = [0, 17, 63]
+        assert np.array_equal(got[sample], oracle.one_to_many(left, right[sample], threads=4))

@@ -193,8 +193,8 @@ FIVE_CONFIGURATIONS = [
     # family, cols, rows, n_left, n_right (per left matrix for n_to_mn), dtype, kernel of the default launch on an MI355X
     ("grouped_overlap", 64, 64, 1, 1, np.float32, "grouped_overlap/pair_in_lds_f32_a1"),
     ("grouped_overlap", 1024, 1024, 1, 1, np.float32, "grouped_overlap/f32_m32x32"),
-    ("multimat_right_grouped", 256, 256, 1, 64, np.float32, "multimat_right_grouped/f32_m16x16_r4"),
-    ("multimat_right_grouped", 128, 128, 8, 16, np.float32, "multimat_right_grouped/f32_m16x16_r4"),
+    ("multimat_right_grouped", 256, 256, 1, 64, np.float32, "multimat_right_grouped/f32_m16x16_r4_s4"),
+    ("multimat_right_grouped", 128, 128, 8, 16, np.float32, "multimat_right_grouped/f32_m16x16_r4_s4"),
     ("multimat_both_grouped", 64, 64, 16, 32, np.float64, "multimat_both_grouped/f64_m8x8_l4r4"),
 ]
 
