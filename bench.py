@@ -29,6 +29,8 @@ MEASURED_TRAFFIC = {
     ("C1", "grouped_overlap/pair_in_lds_f32_a1"): (0.34e6 + 0.18e6, "profiles/pair_in_lds_one_to_one_64.md"),
     ("C2", "grouped_overlap/f32_m32x32"): (2.134e9 + 0.339e9, "profiles/mfma_kernel_f32_m32x32_one_to_one_1024.md"),
     ("C2", "grouped_overlap/f32_a8b4"): (2.360e9 + 0.703e9, "profiles/engine_f32_a8b4_one_to_one_1024.md"),
+    ("C3", "multimat_right_grouped/f32_m16x16_r4_s4"): (0.0191e9 + 0.1305e9, "profiles/engine_other_workloads.md"),
+    ("C4", "multimat_right_grouped/f32_m16x16_r4_s4"): (0.0107e9 + 0.0583e9, "profiles/engine_other_workloads.md"),
     ("C3", "multimat_right_grouped/f32_m16x16_r4"): (0.0191e9 + 0.1318e9, "profiles/engine_other_workloads.md"),
     ("C4", "multimat_right_grouped/f32_m16x16_r4"): (0.0107e9 + 0.0607e9, "profiles/engine_other_workloads.md"),
     ("C3", "multimat_right_grouped/f32_m32x8_r4"): (0.0192e9 + 0.0927e9, "profiles/engine_other_workloads.md"),
@@ -369,7 +371,7 @@ def main():
     }
     if result["roofline"]["bound"] == "mfma":
         result["roofline"]["note"] = (
-            "dense fp32 MFMA roofline (v_mfma_f32_32x32x2_f32: the definition's FMAs only, no padding to a GEMM); the peak assumes "
+            "dense fp32 MFMA roofline (v_mfma_f32_32x32x2_f32 / _16x16x4_f32: the definition's FMAs only, no padding to a GEMM); the peak assumes "
             "2.4 GHz, the shader clock under this kernel is 2.35 GHz" if dtype == np.float32 else
             "dense fp64 MFMA roofline (v_mfma_f64_16x16x4_f64)")
     else:
