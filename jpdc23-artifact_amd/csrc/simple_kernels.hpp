@@ -60,9 +60,11 @@ __device__ __forceinline__ void atomic_add_simple(double *p, double v) { unsafeA
 // holds `strip_lefts` result matrices and blockIdx.z walks (group of strip_lefts left matrices, right matrix).
 // STAGE (one left matrix, small matrices): the block first copies the left matrix and, per right matrix, that matrix into
 // LDS and the threads read their elements from there - same products, same order, less latency per load (the kernel is one
-// dependent chain of loads and FMAs per thread; a 24x24 pair: 22.0 -> 18.1 us, and 16.2 us with the last products of a row
-// loaded together instead of one by one; 16x16: 13.8 -> 8.9 us).
-template <typename T, bool ALL_PAIRS, bool STAGE>
+// dependent chain of loads and FMAs per thread; a 24x24 pair: 22.0 -> 18.1 us, and 16.2 us with WIDE_TAIL; 16x16: 13.8 -> 8.9 us).
+// WIDE_TAIL: the last one to seven products of a row are loaded together like a whole group instead of one by one - shorter chains for
+// launches of few blocks (16x16, 2 x 2 matrices: 13.6 -> 11.2 us), more load instructions for launches that fill the device (16x16,
+// 32 x 32 matrices: 63 -> 93 us): the launcher sets it for launches of at most one block per CU.
+template <typename T, bool ALL_PAIRS, bool STAGE, bool WIDE_TAIL>
 __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__ left, const T *__restrict__ right,
                                                             T *__restrict__ out, int W, int H, int n_left, int batch, int strip_lefts) {
     extern __shared__ __attribute__((aligned(16))) unsigned char overlap_smem[];
@@ -112,7 +114,9 @@ __global__ __launch_bounds__(256) void overlap_wise_kernel(const T *__restrict__
 #pragma unroll
                 for (int i = 0; i < 8; ++i) sum += a[i] * c[i];
             }
-            if (xl < xl_hi) { // the last one to seven products: loaded together like a whole group (from addresses inside the row), added in order
+            if (!WIDE_TAIL) {
+                for (; xl < xl_hi; ++xl) sum += rrow[xl] * lrow[xl];
+            } else if (xl < xl_hi) { // the last one to seven products: loaded together (from addresses inside the row), added in order
                 T a[8], c[8];
 #pragma unroll
                 for (int i = 0; i < 7; ++i) {
@@ -149,15 +153,26 @@ int run_overlap_wise(const T *left, const T *right, T *out, unsigned cols, unsig
         if ((unsigned long long)n_left * batch > 0x7fffffffULL) return fail(XCORR_ERR_INVALID_ARGUMENT, "too many matrices: %u left, %u right", n_left, batch);
     }
     dim3 grid((unsigned)((strip + block.x - 1) / block.x), (Sy + block.y - 1) / block.y, (unsigned)(steps < 65535 ? steps : 65535));
-    // one left matrix and a pair fits 64 KB of LDS: staged (the loops over right matrices per block stay short: gridDim.z covers them)
+    // One left matrix and a pair that fits 64 KB of LDS: staged - always up to 32x32 fp32 (1 x 4000 of 32x32: 4.1 -> 2.7 ms), larger pairs
+    // while the launch has at most sixteen blocks per CU (1 x 32 of 64x64: 491 -> 398 us; 1 x 4000 of 64x64, where the 32 KB per block cost
+    // more occupancy than the shorter loads give back: 32.8 -> 35.7 ms, so not there).
+    const unsigned long long blocks = (unsigned long long)grid.x * grid.y * grid.z;
     const size_t pair_bytes = 2 * (size_t)cols * rows * sizeof(T);
-    const bool stage = n_left == 1 && pair_bytes <= 64 * 1024;
-    if (stage)
-        overlap_wise_kernel<T, false, true><<<grid, block, pair_bytes, stream>>>(left, right, out, (int)cols, (int)rows, 1, (int)batch, 1);
+    const bool stage = n_left == 1 && pair_bytes <= 64 * 1024 && (pair_bytes <= 8 * 1024 || blocks <= 16ull * (unsigned)device_cus());
+    const bool few_blocks = blocks <= (unsigned long long)device_cus();
+    const int W = (int)cols, H = (int)rows, nl = (int)n_left, nb = (int)batch, sl = (int)strip_lefts;
+    if (stage && few_blocks)
+        overlap_wise_kernel<T, false, true, true><<<grid, block, pair_bytes, stream>>>(left, right, out, W, H, 1, nb, 1);
+    else if (stage)
+        overlap_wise_kernel<T, false, true, false><<<grid, block, pair_bytes, stream>>>(left, right, out, W, H, 1, nb, 1);
+    else if (all_pairs && few_blocks)
+        overlap_wise_kernel<T, true, false, true><<<grid, block, 0, stream>>>(left, right, out, W, H, nl, nb, sl);
     else if (all_pairs)
-        overlap_wise_kernel<T, true, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
+        overlap_wise_kernel<T, true, false, false><<<grid, block, 0, stream>>>(left, right, out, W, H, nl, nb, sl);
+    else if (few_blocks)
+        overlap_wise_kernel<T, false, false, true><<<grid, block, 0, stream>>>(left, right, out, W, H, nl, nb, sl);
     else
-        overlap_wise_kernel<T, false, false><<<grid, block, 0, stream>>>(left, right, out, (int)cols, (int)rows, (int)n_left, (int)batch, (int)strip_lefts);
+        overlap_wise_kernel<T, false, false, false><<<grid, block, 0, stream>>>(left, right, out, W, H, nl, nb, sl);
     XCORR_HIP(hipGetLastError());
     xcorr_launch_record &rec = last_launch();
     memset(&rec, 0, sizeof(rec));
