@@ -437,10 +437,17 @@ template <typename T, int A, int B, int U, int COLS>
 __global__ __launch_bounds__(1024) void pair_in_lds_kernel(const T *__restrict__ left_all, const T *__restrict__ right_all, T *__restrict__ out_all,
                                                            const PairGeometry geo) {
     const int W = COLS ? COLS : geo.W, H = geo.H, tasks_x = geo.tasks_x, total_tasks = geo.total_tasks;
-    const int pair = (int)blockIdx.x / geo.blocks_per_pair, block_of_pair = (int)blockIdx.x % geo.blocks_per_pair;
-    const T *left = left_all + (size_t)(pair / geo.left_div) * W * H;
-    const T *right = right_all + (size_t)(geo.right_mod ? pair % geo.right_mod : pair) * W * H;
-    T *out = out_all + (size_t)pair * (2 * W - 1) * (2 * H - 1);
+    // (one pair: no divisions - they would be a twentieth of this kernel's run time on a 16x16 pair)
+    int block_of_pair = (int)blockIdx.x;
+    const T *left = left_all, *right = right_all;
+    T *out = out_all;
+    if ((int)gridDim.x != geo.blocks_per_pair) {
+        const int pair = (int)blockIdx.x / geo.blocks_per_pair;
+        block_of_pair = (int)blockIdx.x - pair * geo.blocks_per_pair;
+        left += (size_t)(pair / geo.left_div) * W * H;
+        right += (size_t)(geo.right_mod ? pair % geo.right_mod : pair) * W * H;
+        out += (size_t)pair * (2 * W - 1) * (2 * H - 1);
+    }
     const int pitch_l = COLS ? COLS + 2 * (B < 16 / (int)sizeof(T) ? 16 / (int)sizeof(T) : B) : geo.pitch_l, pitch_r = COLS ? COLS : geo.pitch_r;
     using vec = typename vec128<T>::type;
     constexpr int VK = 16 / (int)sizeof(T);
