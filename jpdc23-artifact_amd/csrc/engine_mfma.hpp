@@ -7,24 +7,26 @@
 //     i <-> (right matrix u_i, y shift sy_i):   Ua[i][k] = U_{u_i}[yl - sy_i][x_k]      (a window of right rows)
 //     j <-> (left matrix v_j, x shift sx_j):    Vb[k][j] = V_{v_j}[yl][x_k + sx_j]      (a Hankel matrix of one left row)
 // so the whole reduction over (yl, xr) accumulates into the same P x P result tile of v_mfma_f32_32x32x2_f32 (P = 32,
-// two k slots) or v_mfma_f64_16x16x4_f64 (P = 16, four k slots). Nothing is multiplied that the definition does not
-// multiply, except the zero padding at tile edges that the register-tile sweep has as well. Both instructions run at
-// the rate of the vector FMA peak (64 cycles each on this chip), but one instruction stands for 2048 / 1024 FMAs: the
+// two k slots), v_mfma_f32_16x16x4_f32 or v_mfma_f64_16x16x4_f64 (P = 16, four k slots). Nothing is multiplied that the definition does not
+// multiply, except the zero padding at tile edges that the register-tile sweep has as well. The instructions run at
+// the rate of the vector FMA peak (64 cycles each on this chip; the 16 x 16 fp32 one 32), but one stands for 2048 / 1024 FMAs: the
 // LDS reads and address arithmetic around it weigh little (about two cycles of the matrix pipeline per other
 // instruction issued on the SIMD), the shader clock stays at 2.35 GHz on data that holds the vector-FMA loop at 2.0-2.1,
 // and operand reuse happens inside the matrix core instead of in registers: small shift tiles (many matrices per tile)
 // cost nothing extra.
 //
 // Lane l of a wavefront (p = l % P, kk = l / P) supplies row i = p of Ua and column j = p of Vb for k slot kk. The k
-// slots of the EV instructions of a step (4 for the 32 x 32 fp32 tile, 2 for the 16 x 16 fp64 tile) are assigned
+// slots of the EV instructions of a step (4 for the fp32 tiles, 2 for the fp64 tile) are assigned
 // x_k = x0 + EV * kk + e, e = 0 .. EV-1, so the right operand of a step is ONE aligned LDS read of EV elements per lane
-// and the left operand EV consecutive elements. A step covers 8 right columns with every instruction. The work items
+// and the left operand EV consecutive elements. A step covers 8 right columns with every instruction (16 with the 16 x 16 fp32
+// one). The work items
 // (tiles, chunks of rows and columns, centre-out order), the zero-padded LDS bands and the four wavefronts of a block
-// that share one tile are those of the register-tile sweep (engine.hpp); the staging (BandStager) and the deal of a
-// stage's steps to the wavefronts (mfma_stage) are this file's.
+// that share one tile are those of the register-tile sweep (engine.hpp); the staging by loads that write LDS directly
+// (BandDma), the deal of a stage's steps to the wavefronts (mfma_stage, mfma_stage_fine) and the persistent blocks that take
+// their work items from a queue (mfma_kernel) are this file's.
 //
 // Result layout of the instructions (lane l, accumulator element r): column j = l % P; row i = 8 * (r / 4) + 4 * (l / 32) + r % 4
-// for the fp32 instruction and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs (two
+// for the 32 x 32 fp32 instruction, i = 4 * (l / 16) + r for the 16 x 16 fp32 one and i = 4 * r + l / 16 for the fp64 one. The P lanes of a row are adjacent x shifts: 128-byte runs (two
 // runs of 64 bytes in different result rows for the tiles whose columns hold the x shifts twice, see JYO_ below).
 #pragma once
 
