@@ -22,12 +22,19 @@ using D_8x8_l4r4 = MfmaCfg<double, 2, 2, 1, 2, 1, 2, 12, 32, 4>;
 // bound by their LDS reads.)
 using D_32x32_s16 = MfmaCfg<double, 1, 1, 2, 1, 2, 1, 32, 32, 4, 1, 4, 1, 1>;
 
+// ... and with four right matrices in the rows of a result tile (4 y shifts each), four result tiles down a wavefront: 16 x 16 shifts per block,
+// trimmed along y to 4 at a time. Against D_32x8_r4: 1 x 64 of 128x128 0.666 -> 0.622 ms, 1 x 256 of 64x64 0.224 -> 0.201 ms, n-to-mn 8 x 16 of
+// 128x128 1.274 -> 1.213 ms, level at 256x256. (32 x 16 shifts per block: ahead at 64x64 and 256x256 by 1-3 %, 4 % behind at 128x128; stages of 12 rows:
+// level; of 8 rows: 4-6 % behind. Not compiled.)
+using D_16x16_r4_s4 = MfmaCfg<double, 1, 4, 1, 1, 4, 1, 16, 32, 4, 1, 4, 1, 1>;
+
 static const EngineSpec specs[] = {
     make_spec<D_32x32>("f64_m32x32", 0.696, 1.0),
     make_spec<D_32x16>("f64_m32x16", 0.697, 1.0),
     make_spec<D_32x8_r4>("f64_m32x8_r4", 0.705, 1.0),
     make_spec<D_8x8_l4r4>("f64_m8x8_l4r4", 0.730, 1.0),
     make_spec<D_32x32_s16>("f64_m32x32_s16", 0.80, 1.0),
+    make_spec<D_16x16_r4_s4>("f64_m16x16_r4_s4", 0.73, 1.0),
 };
 
 const EngineSpec *engine_mfma_specs_f64(int *count) {

@@ -74,6 +74,7 @@ static const struct {
     {"f64_m32x8_r4", 4},
     {"f64_m8x8_l4r4", 4},
     {"f64_m32x32_s16", 4},
+    {"f64_m16x16_r4_s4", 3},
 };
 
 int EngineSpec::resident_blocks() const {
