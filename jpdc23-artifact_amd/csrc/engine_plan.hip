@@ -308,6 +308,19 @@ static double predict_us(const EngineSpec &s, const EngineRequest &rq, const Eng
     // register tiles is 1.0 below half a millisecond and 1.3 from five milliseconds on, of the matrix-core tiles 1.1
     // throughout: the register tiles pay the difference, phased in over a decade of run time.
     if (!s.MFMA && t > 500.0) t *= 1.0 + 0.18 * std::fmin(1.0, std::log10(t / 500.0));
+    {
+        // No launch is faster than its multiply instructions. A wavefront of a matrix-core block owns one SIMD's matrix pipeline, 2 (fp64: 4)
+        // cycles per accumulator element and multiplied element pair, the clock holds 2.35 GHz under that kernel and the pipelines measured busy
+        // 0.94 of the time at best (0.92 with the 32-cycle instruction of the tile-by-tile sweeps); the vector-FMA tiles issue in 0.86-0.89 of the
+        // cycles at the 2.0-2.1 GHz their load pulls the clock to: 0.75 of the rate at 2.4 GHz for the A8xB4 tile, the others in proportion to
+        // their issue factors. The fitted terms above are up to 20 % below this bound where many equal items keep every CU in its sweep (C2,
+        // thousands of pairs from 128x128 on, pairs of 4096x4096 and more).
+        const double best_rate = s.MFMA ? (s.fine_x ? 0.93 : 0.95) * 2350.0 / 2400.0 : 0.75 * (f32 ? 0.713 : 0.676) / s.issue_factor;
+        const double multiplies = (double)s.NV * s.NU * s.A * s.B / s.WZ * (rows_avg - window) * cols_avg; // per wavefront of an average item
+        // (plans at the bound still differ by what the fitted terms see - chunk sizes, atomic adds -: a small share of them keeps their order)
+        const double bound = items * multiplies * (f32 ? 2.0 : 4.0) / 2400.0 / cus / best_rate + (split ? (plan.ordered ? 0.0 : t_clear) : 0.0);
+        if (bound > t) t = bound + 0.03 * t;
+    }
     return t;
 }
 
