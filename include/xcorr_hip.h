@@ -265,8 +265,8 @@ int xcorr_block_per_overlap_f64(const double *left, const double *right, double 
 
 /* Few small matrices. A launch is short of work for 256 CUs when its matrices are few and small, and what it costs then is
  * the number of kernels it takes and the latency of one block. xcorr_shuffle, xcorr_split_row, xcorr_multimat_right(_groups),
- * xcorr_multimat_both, xcorr_grouped_overlap, the work-distribution variant of xcorr_warp_per_overlap and
- * xcorr_warp_per_overlap_lds therefore hand such a launch to one kernel of another kind when the call names no tile, no
+ * xcorr_multimat_both, xcorr_grouped_overlap, xcorr_multimat_right_grouped, xcorr_multimat_both_grouped, the work-distribution
+ * variant of xcorr_warp_per_overlap and xcorr_warp_per_overlap_lds therefore hand such a launch to one kernel of another kind when the call names no tile, no
  * chunk of rows or columns and none of the LDS family's staging sizes: every block keeps both matrices of ITS pair whole in
  * LDS and its wavefronts reduce groups of four adjacent x shifts over all rows (the role of run_ccn_warp_per_shift_shared_mem,
  * kernels.cuh:144-161, at such sizes). One launch, plain stores, the same bits every run: `out` need not be zeroed whatever

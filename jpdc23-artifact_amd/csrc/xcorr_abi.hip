@@ -403,6 +403,13 @@ int multimat_right_grouped_impl(const T *left, const T *right, T *out, unsigned 
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::combined))) return rc;
     if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::combined))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, (size_t)n_left * n_right), cols, rows, (size_t)n_left * n_right, &rc)) {
+        PairList pairs;
+        pairs.n_pairs = n_left * n_right;
+        pairs.left_div = n_right; // left l meets the right matrices [l * n_right, (l + 1) * n_right)
+        return run_pair_in_lds<T>("multimat_right_grouped", left, right, out, cols, rows, as_stream(stream), pairs);
+    }
+    if (rc) return rc;
     EngineRequest rq = base_request("multimat_right_grouped", sizeof(T), left, right, out, cols, rows, n_left,
                                     n_left * n_right, p);
     rq.group_m = n_left > 1 ? (int)n_right : 0;
@@ -461,6 +468,14 @@ int multimat_both_grouped_impl(const T *left, const T *right, T *out, unsigned c
     if ((rc = check_limit("right matrices per thread", p.right_matrices_per_thread, Limits::combined))) return rc;
     if ((rc = check_limit("left rows per iteration", p.left_rows_per_iteration, Limits::combined))) return rc;
     if ((rc = check_dist(p.distribution_type))) return rc;
+    if (small_pairs_in_lds<T>(p, names_tile_or_chunk(p, (size_t)n_left * n_right), cols, rows, (size_t)n_left * n_right, &rc)) {
+        PairList pairs;
+        pairs.n_pairs = n_left * n_right;
+        pairs.left_div = n_right; // result l * n_right + r
+        pairs.right_mod = n_right;
+        return run_pair_in_lds<T>("multimat_both_grouped", left, right, out, cols, rows, as_stream(stream), pairs);
+    }
+    if (rc) return rc;
     EngineRequest rq = base_request("multimat_both_grouped", sizeof(T), left, right, out, cols, rows, n_left, n_right, p);
     rq.y_shifts = p.shifts_per_thread_right_matrix == 1 ? 2 : p.shifts_per_thread_right_matrix;
     rq.left_mats = p.left_matrices_per_thread;

@@ -214,20 +214,22 @@ def test_few_small_pairs_whole_in_lds(oracle, dtype):
                 # groups: left l against its own n_right right matrices
                 exp = np.concatenate([oracle.one_to_many(l[i:i + 1], r[i * n_right:(i + 1) * n_right]) for i in range(n_left)])
                 family = "multimat_right_groups" if n_left > 1 else "multimat_right"
-                for kw in ({}, dict(distribution_type="triangle")):
-                    got, rec = run_as_planned(xc, family, l, r, n_left * n_right, n_left, n_right, xc.make_params(**kw))
+                for fam, kw in ((family, {}), (family, dict(distribution_type="triangle")), ("multimat_right_grouped", {})):
+                    got, rec = run_as_planned(xc, fam, l, r, n_left * n_right, n_left, n_right, xc.make_params(**kw))
                     assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
-                    check(got, exp, exact, f"{family} {kw} {n_left}x{n_right} {shape}")
+                    check(got, exp, exact, f"{fam} {kw} {n_left}x{n_right} {shape}")
                 # all pairs: every left against the first n_right right matrices
                 exp = oracle.n_to_m(l, r[:n_right])
-                got, rec = run_as_planned(xc, "multimat_both", l, r[:n_right], n_left * n_right, n_left, n_right, xc.make_params())
-                assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
-                check(got, exp, exact, f"multimat_both {n_left}x{n_right} {shape}")
+                for fam in ("multimat_both", "multimat_both_grouped"):
+                    got, rec = run_as_planned(xc, fam, l, r[:n_right], n_left * n_right, n_left, n_right, xc.make_params())
+                    assert "pair_in_lds" in rec["kernel"] and rec["uses_atomics"] == 0, rec
+                    check(got, exp, exact, f"{fam} {n_left}x{n_right} {shape}")
     # what keeps the engine: a chunk or a tile named, whole_pair_in_lds = 2, more than 64 pairs, matrices beyond 32 x 32
     left, right = ints(rng, (8, 16, 16), dtype), ints(rng, (72, 16, 16), dtype)
     for family, n_left, n_right, kw in [("multimat_both", 8, 8, dict(rows_per_thread=8)), ("multimat_both", 8, 8, dict(whole_pair_in_lds=2)),
                                         ("multimat_both", 8, 8, dict(left_matrices_per_thread=2)), ("multimat_both", 8, 9, {}),
-                                        ("multimat_right", 1, 72, {}), ("multimat_right", 1, 8, dict(right_matrices_per_thread=2))]:
+                                        ("multimat_right", 1, 72, {}), ("multimat_right", 1, 8, dict(right_matrices_per_thread=2)),
+                                        ("multimat_both_grouped", 8, 8, dict(shifts_per_thread_right_matrix=4)), ("multimat_both_grouped", 8, 9, {})]:
         got, rec = run_as_planned(xc, family, left[:n_left], right[:n_right], n_left * n_right, n_left, n_right, xc.make_params(**kw))
         assert "pair_in_lds" not in rec["kernel"], (family, kw, rec)
         exp = oracle.n_to_m(left[:n_left], right[:n_right])
