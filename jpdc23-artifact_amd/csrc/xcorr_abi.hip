@@ -516,7 +516,7 @@ int warp_per_overlap_lds_impl(const T *left, const T *right, T *out, unsigned co
     int rc = check_shape(left, right, out, cols, rows);
     if (rc) return rc;
     const bool named = p.shifts_per_thread_block || p.shared_mem_rows || p.shared_mem_row_size || p.right_matrices_per_block || p.column_group_per_block;
-    if (n_right > 0 && n_right <= 64 && small_pairs_in_lds<T>(p, named, cols, rows, n_right, &rc)) {
+    if (n_right > 0 && small_pairs_in_lds<T>(p, named, cols, rows, n_right, &rc)) {
         PairList pairs;
         pairs.n_pairs = pairs.left_div = n_right;
         return run_pair_in_lds<T>("warp_per_overlap_lds", left, right, out, cols, rows, as_stream(stream), pairs);

@@ -248,9 +248,8 @@ def test_tiles_swept_result_tile_by_result_tile(oracle, dtype):
     got = xc.run("multimat_right_grouped", left, right, 600, n_left=600, n_right=1)
     assert xc.last_launch()["kernel"].endswith("_s16"), xc.last_launch()["kernel"]
     assert np.array_equal(got, oracle.n_to_mn(left, right, threads=8))
-    if True:
-        left, right = ints(rng, (1, 128, 128), dtype), ints(rng, (64, 128, 128), dtype)
-        got = xc.run("multimat_right_grouped", left, right, 64, n_left=1, n_right=64)
-        assert xc.last_launch()["kernel"].endswith("_r4_s4"), xc.last_launch()["kernel"]
-        sample = [0, 17, 63]
-        assert np.array_equal(got[sample], oracle.one_to_many(left, right[sample], threads=4))
+    left, right = ints(rng, (1, 128, 128), dtype), ints(rng, (64, 128, 128), dtype)
+    got = xc.run("multimat_right_grouped", left, right, 64, n_left=1, n_right=64)
+    assert xc.last_launch()["kernel"].endswith("_r4_s4"), xc.last_launch()["kernel"]
+    sample = [0, 17, 63]
+    assert np.array_equal(got[sample], oracle.one_to_many(left, right[sample], threads=4))

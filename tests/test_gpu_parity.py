@@ -245,6 +245,14 @@ def test_few_small_pairs_whole_in_lds(oracle, dtype):
         got, rec = run_as_planned(xc, "warp_per_overlap_lds", left, right, 8, 1, 8, xc.make_params(**kw))
         assert ("pair_in_lds" in rec["kernel"]) == routed, (kw, rec)
         check(got, oracle.one_to_many(left, right), True, f"warp_per_overlap_lds {kw}")
+    # forced (whole_pair_in_lds = 1): also beyond the sizes the launcher would pick it for
+    left, right = ints(rng, (3, 20, 36), dtype), ints(rng, (70, 20, 36), dtype)
+    got, rec = run_as_planned(xc, "multimat_both", left, right, 210, 3, 70, xc.make_params(whole_pair_in_lds=1))
+    assert "pair_in_lds" in rec["kernel"], rec
+    check(got, oracle.n_to_m(left, right), True, "forced multimat_both 3x70")
+    got, rec = run_as_planned(xc, "warp_per_overlap_lds", left[:1], right, 70, 1, 70, xc.make_params(whole_pair_in_lds=1))
+    assert "pair_in_lds" in rec["kernel"], rec
+    check(got, oracle.one_to_many(left[:1], right), True, "forced warp_per_overlap_lds 1x70")
 
 
 ONE_TO_MANY_CASES = [
